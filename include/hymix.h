@@ -71,31 +71,49 @@ int hm_relu_squared(int dtype, const void* z, int64_t z_stride, void* out, int64
  *   unit_norm: every rotated head divided by its RMS;
  *   v_first != NULL: v <- (1 - lam[0]) v + lam[0] v_first[t];
  *   k and v go to row slot_mapping[t] of the caches [rows, G, D] / [rows, G, V] (a negative row: not stored);
- *   q_out [T, H, D]. */
+ *   q_out [T, H, D].
+ * q_head_w / k_head_w != NULL ([D], one row shared by the heads): before the rotation every q (k) head is divided by its
+ * own RMS and multiplied by that row; q_head_scale != NULL (f32 [H]): query head h times q_head_scale[h] after it.
+ * k_cache == v_cache == NULL: the rows hold q only (keys and values are another layer's), nothing is stored. */
 int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, int H, int G, int D, int V, const void* q_norm_w,
                    const void* k_norm_w, float eps, const float* inv_freq, int rot_half, int unit_norm, const int32_t* tok_pos,
                    const int32_t* slot_mapping, void* k_cache, void* v_cache, const void* v_first, int64_t v_first_stride,
-                   const float* lam, void* q_out, int64_t T, void* stream);
+                   const float* lam, void* q_out, int64_t T, const void* q_head_w, const void* k_head_w,
+                   const float* q_head_scale, void* stream);
 
 /* Attention of q [T, H, D] over the paged caches, any sizes, f32 arithmetic: the token at position i sees key j <= i,
  * and with window > 0 only if i - j < window or j < keep_first.  sink != NULL (f32 [H]): exp(sink[h]) joins the softmax
- * denominator.  o [T, H, V]. */
+ * denominator.  o [T, H, V].
+ * Pooled blocks (pool > 0, needs window > 0 and keep_first == 0): beside its window the token at position i sees one
+ * key and value for every block of `pool` tokens whose last token lies at or before i - window: the block's mean key and
+ * mean value, row e % pool_rows of page block_table[e / pool_rows] of kp_cache [pages, pool_rows, G, D] and vp_cache
+ * [pages, pool_rows, G, V] for block e (pool_rows * pool >= block_size); they share the softmax with the tokens. */
 int hm_attn_rows(int dtype, const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                  const int32_t* tok_seq, const int32_t* tok_pos, const float* sink, int window, int keep_first, float scale,
-                 void* o, int64_t T, int H, int G, int D, int V, int block_size, int max_blocks, void* stream);
+                 void* o, int64_t T, int H, int G, int D, int V, int block_size, int max_blocks, const void* kp_cache,
+                 const void* vp_cache, int pool, int pool_rows, void* stream);
+
+/* For every token of the step whose position ends a block of `pool` tokens: the mean of the block's keys and of its
+ * values, as the caches hold them (f32 sums), written to the pooled caches (layout above).  Launch it after the step's
+ * keys and values are stored. */
+int hm_pool_blocks(int dtype, const void* k_cache, const void* v_cache, void* kp_cache, void* vp_cache,
+                   const int32_t* block_tables, const int32_t* tok_seq, const int32_t* tok_pos, int64_t T, int G, int D, int V,
+                   int block_size, int max_blocks, int pool, int pool_rows, void* stream);
 
 /* The same attention on the matrix cores, bf16 storage only, dim and vdim multiples of 8 up to 128, block_size % 64 == 0.
  * Portions of any length (max_q = the longest portion of the step): */
 int hm_attn_tiles(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables, const int32_t* qstart,
                   const int32_t* seq_pos0, const float* sink, int window, int keep_first, float scale, void* o, int B, int max_q,
-                  int H, int G, int D, int V, int block_size, int max_blocks, void* stream);
+                  int H, int G, int D, int V, int block_size, int max_blocks, const void* kp_cache, const void* vp_cache, int pool,
+                  int pool_rows, void* stream);
 /* Single-token queries (q [B, H, D], ctx[b] = keys of sequence b incl. the new one): the visible key tiles are split
  * over `splits` workgroups per (sequence, key/value head) and merged in split order by a second launch.  At most 32
  * query heads per key/value head.  workspace: hm_attn_decode_workspace_bytes(B, H, V, splits) bytes. */
 size_t hm_attn_decode_workspace_bytes(int64_t B, int H, int V, int splits);
 int hm_attn_decode(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables, const int32_t* ctx,
                    const float* sink, int window, int keep_first, float scale, void* o, int64_t B, int H, int G, int D, int V,
-                   int block_size, int max_blocks, int splits, void* workspace, size_t workspace_bytes, void* stream);
+                   int block_size, int max_blocks, int splits, void* workspace, size_t workspace_bytes, const void* kp_cache,
+                   const void* vp_cache, int pool, int pool_rows, void* stream);
 
 /* prep [T, H, 5, D] f32 = decay | a*u | u | k | r from the columns r_off, k_off, a_off (H*D wide) and z_off (rank wide) of
  * proj:  decay = exp(-decay_scale * sigmoid(w2 tanh(z) + w0)), a = sigmoid(a_pre + a_bias), u = k / sqrt(sum k^2 + unit_eps)
@@ -115,6 +133,18 @@ int hm_delta_recurrence(int dtype, const float* prep, const void* v, int64_t v_s
 /* out[t, h*D + i] = o[t, h, i] / sqrt(mean_i o[t, h]^2 + eps) * norm_w[h*D + i] * sigmoid(g[t, h*D + i]). */
 int hm_delta_gate_norm(int dtype, const float* o, const void* g, int64_t g_stride, const void* norm_w, float eps, void* out,
                        int64_t T, int H, int D, void* stream);
+
+/* The boundary between two sublayers of a residual that is normalised on the sublayers' OUTPUT, with an RMS norm over
+ * `groups` equal consecutive parts of the vector (each part divided by its own sqrt(mean(part^2) + eps)); x [T, W] f32 is
+ * updated in place, per token in one launch:
+ *   y != NULL, ids == NULL:  x[t] += group_norm(y[t]) * post_w
+ *   y != NULL, ids != NULL:  x[t]  = group_norm(y[ids[t]]) * post_w       (y = an embedding table)
+ *   h_out != NULL:           h_out[t] = next_w ? group_norm(x[t]) * next_w : x[t], in the storage type. */
+int hm_group_norm_residual(int dtype, float* x, const void* y, const int64_t* ids, const void* post_w, const void* next_w,
+                           int groups, float eps, void* h_out, int64_t T, int W, void* stream);
+
+/* x[i] <- cap * tanh(x[i] * scale / cap) (cap <= 0: x[i] * scale), f32 in place. */
+int hm_scale_softcap(float* x, int64_t n, float scale, float cap, void* stream);
 
 #ifdef __cplusplus
 }

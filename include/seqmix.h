@@ -25,6 +25,13 @@ extern "C" {
 #define SM_F32 0
 #define SM_BF16 1
 
+#define SM_ROUTE_SOFTMAX 0
+#define SM_ROUTE_SIGMOID 1
+
+#define SM_ACT_CLAMPED_GLU 0
+#define SM_ACT_GELU 1
+#define SM_ACT_GELU_TANH 2
+
 #define SM_OK 0
 #define SM_EINVAL (-1)
 #define SM_ESHAPE (-2)
@@ -70,14 +77,26 @@ int sm_latent_norm_store(int dtype, const void* x, int64_t row_stride, const voi
  * The portable kernel (any R, both storage types): one workgroup per (token, head). */
 int sm_latent_attn_rows(int dtype, const void* q, const void* cache, const int32_t* block_tables, const int32_t* tok_seq,
                         const int32_t* tok_pos, void* o, float scale, int64_t T, int H, int R, int block_size,
-                        int max_blocks, void* stream);
+                        int max_blocks, int RV, int window, void* stream);
+/* In the three attention calls: RV > 0 = only the first RV columns of a cache row are values (the rest, e.g. a rotated
+ * key part, only enters the scores) and o is [T, H, RV]; RV <= 0 = R.  window > 0: the token at position i sees only the
+ * keys j with i - j < window. */
+
+/* A latent with a rotated key part: x rows (x_stride apart) hold [R | Rd]; c = rms_norm(x[:R]) * w and x[R:] with its
+ * first rot_dims channels turned by tok_pos * inv_freq[i] (channel 2i with 2i + 1, f32 angles) go to cache row
+ * slot_mapping[t] of a paged cache [rows, R + Rd].  q rows (q_stride apart) hold per head [D | Rd]; every head's Rd part
+ * is turned the same way and written to columns R .. R + Rd of qa [T, H, R + Rd] (whose first R columns, the absorbed
+ * queries, are the caller's). */
+int sm_latent_rope_store(int dtype, const void* x, int64_t x_stride, const void* w, float eps, const void* q, int64_t q_stride,
+                         void* qa, const float* inv_freq, int rot_dims, const int32_t* tok_pos, void* cache,
+                         const int32_t* slot_mapping, int64_t T, int H, int D, int R, int Rd, void* stream);
 
 /* The same product on the matrix cores (bf16, R % 8 == 0, R <= 256, block_size % 64 == 0): a workgroup owns 128
  * consecutive (token, head) rows of one sequence and walks 64-key tiles of the cache.  qstart [B + 1]; seq_pos0[b]
  * = position of the sequence's first token in this step; max_q = the longest portion.  */
 int sm_latent_attn_tiles(const void* q, const void* cache, const int32_t* block_tables, const int32_t* qstart,
                          const int32_t* seq_pos0, void* o, float scale, int B, int max_q, int H, int R, int block_size,
-                         int max_blocks, void* stream);
+                         int max_blocks, int RV, int window, void* stream);
 
 /* Single-token queries (decode) on the matrix cores with the keys split over workgroups: every (sequence, split)
  * writes an unnormalised partial state to `workspace`, a second launch merges them.  ctx[b] = keys visible to the
@@ -85,7 +104,7 @@ int sm_latent_attn_tiles(const void* q, const void* cache, const int32_t* block_
 size_t sm_latent_decode_workspace_bytes(int64_t B, int H, int R, int splits);
 int sm_latent_attn_decode(const void* q, const void* cache, const int32_t* block_tables, const int32_t* ctx, void* o,
                           float scale, int64_t B, int H, int R, int block_size, int max_blocks, int splits,
-                          void* workspace, size_t workspace_bytes, void* stream);
+                          void* workspace, size_t workspace_bytes, int RV, int window, void* stream);
 
 /* PolyNorm: out = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over the F columns of a row;
  * coef = {a, b, c, e} f32 on the device. */
@@ -98,14 +117,19 @@ int sm_clamped_glu(int dtype, const void* gu, float limit, float alpha, void* ou
 /* Router: z = router_w h (f32), s = softmax(z) over E experts; experts form `groups` equal groups of neighbours, a
  * group scores its largest s, only experts of the best `keep` groups are eligible (groups <= 1: all are); the `top`
  * eligible experts with the largest s are chosen, weights = their s / (sum + 1e-20).  idx [T, top] i32, wts [T, top] f32. */
+/* score = SM_ROUTE_SIGMOID: s = sigmoid(z) instead.  correction != NULL (f32 [E]): the choice (groups and experts) goes
+ * by s + correction, the weights stay s.  group_top (1..4): a group scores the sum of its group_top largest choice
+ * scores.  renorm == 0: the weights are the chosen s as they are. */
 int sm_moe_route(int dtype, const void* h, const float* router_w, int32_t* idx, float* wts, int64_t T, int W, int E,
-                 int top, int groups, int keep, void* stream);
+                 int top, int groups, int keep, int score, const float* correction, int group_top, int renorm, void* stream);
 
 /* Expert products, one (token, chosen expert) pair at a time (memory-bound form for few tokens):
  * act[p] = clamped_glu(w_gu[e] h[t]) with w_gu [E, 2F, W] (gate rows, then up rows), p = t * top + k; then
  * y[t] = sum_k wts[t, k] * (w_down[e_k] act[t * top + k]) + shared[t]   (w_down [E, W, F]; shared may be NULL). */
+/* act_kind = SM_ACT_CLAMPED_GLU as above; SM_ACT_GELU / SM_ACT_GELU_TANH: an expert is w_down act(w_up h) with the exact
+ * (erf) or the tanh GELU, and w_gu is [E, F, W] (one part when tiled). */
 int sm_moe_pairs_gate_up(int dtype, const void* h, const int32_t* idx, const void* w_gu, float limit, float alpha,
-                         void* act, int64_t T, int top, int W, int F, void* stream);
+                         int act_kind, void* act, int64_t T, int top, int W, int F, void* stream);
 int sm_moe_pairs_down(int dtype, const void* act, const int32_t* idx, const float* wts, const void* w_down,
                       const void* shared, void* y, int64_t T, int top, int W, int F, void* stream);
 
@@ -116,7 +140,7 @@ int sm_moe_pairs_down(int dtype, const void* act, const int32_t* idx, const floa
  * tile_expert int32 [n], pair_row int32 [T * top], act bf16 [32 n, F], prod bf16 [32 n, W]. */
 int sm_moe_grouped_tiles(int64_t T, int top, int E);
 int sm_moe_grouped(const void* h, const int32_t* idx, const float* wts, const void* w_gu, const void* w_down,
-                   const void* shared, float limit, float alpha, void* y, int64_t T, int top, int E, int W, int F,
+                   const void* shared, float limit, float alpha, int act_kind, void* y, int64_t T, int top, int E, int W, int F,
                    int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row, void* act, void* prod, void* stream);
 
 /* sm_moe_grouped with tiles of 128 rows (activations of a tile staged once in LDS, every weight fragment reused by four
@@ -124,7 +148,7 @@ int sm_moe_grouped(const void* h, const int32_t* idx, const float* wts, const vo
  * row_pair int32 [128 n], tile_expert int32 [n], pair_row int32 [T * top], act bf16 [128 n, F], prod bf16 [128 n, W]. */
 int sm_moe_tiles128_count(int64_t T, int top, int E);
 int sm_moe_tiles128(const void* h, const int32_t* idx, const float* wts, const void* w_gu, const void* w_down,
-                    const void* shared, float limit, float alpha, void* y, int64_t T, int top, int E, int W, int F,
+                    const void* shared, float limit, float alpha, int act_kind, void* y, int64_t T, int top, int E, int W, int F,
                     int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row, void* act, void* prod, void* stream);
 
 /* The two ends of sm_moe_grouped on their own (bf16): the grouping (same scratch layout) and the weighted sum of a token's

@@ -10,6 +10,8 @@ namespace hm {
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ qkv, int64_t row_stride, int H, int G, int D,
                                                           int V, const T* __restrict__ q_norm_w, const T* __restrict__ k_norm_w,
+                                                          const T* __restrict__ q_head_w, const T* __restrict__ k_head_w,
+                                                          const float* __restrict__ q_head_scale,
                                                           float eps, const float* __restrict__ inv_freq, int rot_half,
                                                           int unit_norm, const int32_t* __restrict__ tok_pos,
                                                           const int32_t* __restrict__ slot_mapping, T* __restrict__ k_cache,
@@ -20,6 +22,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ 
     __shared__ float red[16];
     const int64_t t = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (k_cache == nullptr) G = 0;             // the row holds q only: keys and values come from another layer's cache
     const int nq = H * D, nk = G * D, nv = G * V;
     struct alignas(sizeof(T) * VEC) Pack { T v[VEC]; };
     const T* row = qkv + (size_t)t * row_stride;
@@ -41,6 +44,24 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ 
         const float rq = 1.f / sqrtf(sq / (float)nq + eps), rk = 1.f / sqrtf(sk / (float)nk + eps);
         for (int c = tid; c < nq + nk; c += 256)
             qk[c] = c < nq ? qk[c] * rq * to_f(q_norm_w[c]) : qk[c] * rk * to_f(k_norm_w[c - nq]);
+    }
+    if (q_head_w != nullptr || q_head_scale != nullptr) {
+        // every head RMS-normalised over its own channels with one weight row shared by the heads (a wave per head);
+        // then the query heads times their own number
+        __syncthreads();
+        for (int hh = wave; hh < H + G; hh += 4) {
+            float* p = qk + (size_t)hh * D;
+            float r = 1.f;
+            if (q_head_w != nullptr) {
+                float ss = 0.f;
+                for (int i = lane; i < D; i += 64) ss += p[i] * p[i];
+                ss = wave_sum(ss);
+                r = 1.f / sqrtf(ss / (float)D + eps);
+            }
+            const T* w = q_head_w == nullptr ? nullptr : (hh < H ? q_head_w : k_head_w);
+            const float hs = (q_head_scale != nullptr && hh < H) ? q_head_scale[hh] : 1.f;
+            for (int i = lane; i < D; i += 64) p[i] = (w ? p[i] * r * to_f(w[i]) : p[i]) * hs;
+        }
     }
     // the angles depend on the channel pair alone: one sine and cosine per pair, shared by all heads
     float* cs = qk + nq + nk;
@@ -108,7 +129,8 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const T* __restrict__ q,
                                                         const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
                                                         const float* __restrict__ sink, int window, int keep_first, float scale,
                                                         T* __restrict__ o, int H, int G, int D, int V, int block_size,
-                                                        int max_blocks) {
+                                                        int max_blocks, const T* __restrict__ kp_cache,
+                                                        const T* __restrict__ vp_cache, int pool, int pool_rows) {
     extern __shared__ float q_lds[];                 // D floats
     __shared__ float s_lds[kRowChunk];
     __shared__ int row_lds[kRowChunk];
@@ -117,7 +139,8 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const T* __restrict__ q,
     const int b = tok_seq[t], n = tok_pos[t] + 1;    // keys 0 .. n-1 are causal
     const int lo = window > 0 ? max(0, n - window) : 0;
     const int kept = window > 0 ? min(keep_first, lo) : 0;
-    const int total = kept + (n - lo);
+    const int seen = pooled_seen(n - 1, window, pool);       // pooled blocks that lie wholly before the window
+    const int total = seen + kept + (n - lo);
     const int32_t* table = block_tables + (size_t)b * max_blocks;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const T* qr = q + ((size_t)t * H + hd) * D;
@@ -128,19 +151,24 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const T* __restrict__ q,
         __syncthreads();                             // q_lds ready / previous chunk's s_lds and row_lds consumed
         if (tid < kRowChunk) {
             const int e = k0 + tid;
-            const int key = e < kept ? e : lo + (e - kept);
-            row_lds[tid] = e < total ? table[key / block_size] * block_size + key % block_size : -1;
+            if (e < seen) {                          // a pooled entry: row -2 - r of the pooled caches
+                row_lds[tid] = -2 - (table[e / pool_rows] * pool_rows + e % pool_rows);
+            } else {
+                const int f = e - seen;
+                const int key = f < kept ? f : lo + (f - kept);
+                row_lds[tid] = e < total ? table[key / block_size] * block_size + key % block_size : -1;
+            }
         }
         __syncthreads();
         for (int kk = wave; kk < kRowChunk; kk += 4) {
             const int row = row_lds[kk];
             float d = 0.f;
-            if (row >= 0) {
-                const T* kr = k_cache + ((size_t)row * G + g) * D;
+            if (row != -1) {
+                const T* kr = row >= 0 ? k_cache + ((size_t)row * G + g) * D : kp_cache + ((size_t)(-2 - row) * G + g) * D;
                 for (int c = lane; c < D; c += 64) d += q_lds[c] * to_f(kr[c]);
             }
             d = wave_sum(d);
-            if (lane == 0) s_lds[kk] = row >= 0 ? d * scale : -INFINITY;
+            if (lane == 0) s_lds[kk] = row != -1 ? d * scale : -INFINITY;
         }
         __syncthreads();
         float mx = m_run;
@@ -150,10 +178,10 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const T* __restrict__ q,
         for (int r = 0; r < 4; ++r) acc[r] *= alpha;
         for (int kk = 0; kk < kRowChunk; ++kk) {
             const int row = row_lds[kk];
-            if (row < 0) break;
+            if (row == -1) break;
             const float p = expf(s_lds[kk] - mx);
             psum += p;
-            const T* vr = v_cache + ((size_t)row * G + g) * V;
+            const T* vr = row >= 0 ? v_cache + ((size_t)row * G + g) * V : vp_cache + ((size_t)(-2 - row) * G + g) * V;
             for (int r = 0; r < 4; ++r) {
                 const int c = tid + 256 * r;
                 if (c < V) acc[r] += p * to_f(vr[c]);
@@ -177,6 +205,35 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const T* __restrict__ q,
     }
 }
 
+// Mean key and mean value of every block of `pool` tokens that a step completes: one workgroup per token; the token
+// whose position ends a block averages the block's rows as the caches hold them (f32 sums) into the pooled caches.
+template <typename T>
+__global__ __launch_bounds__(256) void pool_blocks_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+                                                          T* __restrict__ kp_cache, T* __restrict__ vp_cache,
+                                                          const int32_t* __restrict__ block_tables,
+                                                          const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                                                          int nk, int nv, int block_size, int max_blocks, int pool, int pool_rows) {
+    const int64_t t = blockIdx.x;
+    const int pos = tok_pos[t];
+    if ((pos + 1) % pool != 0) return;
+    const int blk = pos / pool, first = blk * pool;
+    const int32_t* table = block_tables + (size_t)tok_seq[t] * max_blocks;
+    const size_t prow = (size_t)table[blk / pool_rows] * pool_rows + blk % pool_rows;
+    const float inv = 1.f / (float)pool;
+    for (int c = threadIdx.x; c < nk + nv; c += 256) {
+        const bool is_k = c < nk;
+        const T* src = is_k ? k_cache + c : v_cache + (c - nk);
+        const int width = is_k ? nk : nv;
+        float sum = 0.f;
+        for (int j = 0; j < pool; ++j) {
+            const int key = first + j;
+            sum += to_f(src[((size_t)table[key / block_size] * block_size + key % block_size) * width]);
+        }
+        if (is_k) kp_cache[prow * nk + c] = from_f<T>(sum * inv);
+        else vp_cache[prow * nv + (c - nk)] = from_f<T>(sum * inv);
+    }
+}
+
 }  // namespace hm
 
 using namespace hm;
@@ -185,11 +242,13 @@ extern "C" int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, in
                               const void* k_norm_w, float eps, const float* inv_freq, int rot_half, int unit_norm,
                               const int32_t* tok_pos, const int32_t* slot_mapping, void* k_cache, void* v_cache,
                               const void* v_first, int64_t v_first_stride, const float* lam, void* q_out, int64_t T,
-                              void* stream) {
+                              const void* q_head_w, const void* k_head_w, const float* q_head_scale, void* stream) {
+    const bool q_only = !k_cache && !v_cache;
     if (T < 0 || H < 1 || G < 1 || D < 1 || V < 1 || H % G != 0 || rot_half < 0 || 2 * rot_half > D ||
-        row_stride < (int64_t)(H + G) * D + (int64_t)G * V || (!q_norm_w) != (!k_norm_w) || (rot_half > 0 && !inv_freq) ||
-        (v_first && (!lam || v_first_stride < (int64_t)G * V)) ||
-        (T > 0 && (!qkv || !tok_pos || !slot_mapping || !k_cache || !v_cache || !q_out))) {
+        row_stride < (q_only ? (int64_t)H * D : (int64_t)(H + G) * D + (int64_t)G * V) || (!q_norm_w) != (!k_norm_w) ||
+        (rot_half > 0 && !inv_freq) || (v_first && (!lam || v_first_stride < (int64_t)G * V)) || (!k_cache) != (!v_cache) ||
+        (q_only && (v_first || k_norm_w)) || (q_head_w && !q_only && !k_head_w) ||
+        (T > 0 && (!qkv || !tok_pos || !slot_mapping || !q_out))) {
         set_error("hm_qkv_prepare: bad argument");
         return HM_EINVAL;
     }
@@ -197,12 +256,14 @@ extern "C" int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, in
     if (lds > 60 * 1024) { set_error("hm_qkv_prepare: (heads + kv_heads) * dim = %d does not fit the row buffer", (H + G) * D); return HM_ESHAPE; }
     if (T == 0) return HM_OK;
     // packs need every segment (q, k, v, the rows themselves and the blended values' rows) on multiples of 8 elements
+    if (q_only) G = 0;
     const bool wide = (H * D) % 8 == 0 && (G * D) % 8 == 0 && (G * V) % 8 == 0 && row_stride % 8 == 0 &&
                       (!v_first || v_first_stride % 8 == 0);
     const uintptr_t bits = (uintptr_t)qkv | (uintptr_t)v_first | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)v_cache;
 #define HM_PREP(VEC_)                                                                                                         \
     hipLaunchKernelGGL((qkv_prepare_kernel<DT, VEC_>), dim3((unsigned)T), dim3(256), lds, as_stream(stream), (const DT*)qkv,  \
-                       row_stride, H, G, D, V, (const DT*)q_norm_w, (const DT*)k_norm_w, eps, inv_freq, rot_half, unit_norm,  \
+                       row_stride, H, G, D, V, (const DT*)q_norm_w, (const DT*)k_norm_w, (const DT*)q_head_w,                 \
+                       (const DT*)k_head_w, q_head_scale, eps, inv_freq, rot_half, unit_norm,                                 \
                        tok_pos, slot_mapping, (DT*)k_cache, (DT*)v_cache, (const DT*)v_first, v_first_stride, lam, (DT*)q_out)
     HM_DISPATCH(dtype, "hm_qkv_prepare", if (wide && bits % (8 * sizeof(DT)) == 0) HM_PREP(8); else HM_PREP(1));
 #undef HM_PREP
@@ -213,8 +274,9 @@ extern "C" int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, in
 extern "C" int hm_attn_rows(int dtype, const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                             const int32_t* tok_seq, const int32_t* tok_pos, const float* sink, int window, int keep_first,
                             float scale, void* o, int64_t T, int H, int G, int D, int V, int block_size, int max_blocks,
-                            void* stream) {
+                            const void* kp_cache, const void* vp_cache, int pool, int pool_rows, void* stream) {
     if (T < 0 || H < 1 || G < 1 || H % G != 0 || D < 1 || V < 1 || block_size < 1 || max_blocks < 1 || window < 0 || keep_first < 0 ||
+        pool < 0 || (pool > 0 && (!kp_cache || !vp_cache || window < 1 || keep_first > 0 || pool_rows * pool < block_size)) ||
         (T > 0 && (!q || !k_cache || !v_cache || !block_tables || !tok_seq || !tok_pos || !o))) {
         set_error("hm_attn_rows: bad argument");
         return HM_EINVAL;
@@ -225,7 +287,26 @@ extern "C" int hm_attn_rows(int dtype, const void* q, const void* k_cache, const
     HM_DISPATCH(dtype, "hm_attn_rows",
                 hipLaunchKernelGGL(attn_rows_kernel<DT>, grid, dim3(256), (size_t)D * 4, as_stream(stream), (const DT*)q,
                                    (const DT*)k_cache, (const DT*)v_cache, block_tables, tok_seq, tok_pos, sink, window,
-                                   keep_first, scale, (DT*)o, H, G, D, V, block_size, max_blocks));
+                                   keep_first, scale, (DT*)o, H, G, D, V, block_size, max_blocks, (const DT*)kp_cache,
+                                   (const DT*)vp_cache, pool, pool_rows));
     HM_CHECK_LAUNCH("hm_attn_rows");
+    return HM_OK;
+}
+
+extern "C" int hm_pool_blocks(int dtype, const void* k_cache, const void* v_cache, void* kp_cache, void* vp_cache,
+                              const int32_t* block_tables, const int32_t* tok_seq, const int32_t* tok_pos, int64_t T, int G, int D,
+                              int V, int block_size, int max_blocks, int pool, int pool_rows, void* stream) {
+    if (T < 0 || G < 1 || D < 1 || V < 1 || block_size < 1 || max_blocks < 1 || pool < 1 || pool_rows < 1 ||
+        (int64_t)pool_rows * pool < block_size ||
+        (T > 0 && (!k_cache || !v_cache || !kp_cache || !vp_cache || !block_tables || !tok_seq || !tok_pos))) {
+        set_error("hm_pool_blocks: bad argument");
+        return HM_EINVAL;
+    }
+    if (T == 0) return HM_OK;
+    HM_DISPATCH(dtype, "hm_pool_blocks",
+                hipLaunchKernelGGL(pool_blocks_kernel<DT>, dim3((unsigned)T), dim3(256), 0, as_stream(stream), (const DT*)k_cache,
+                                   (const DT*)v_cache, (DT*)kp_cache, (DT*)vp_cache, block_tables, tok_seq, tok_pos, G * D, G * V,
+                                   block_size, max_blocks, pool, pool_rows));
+    HM_CHECK_LAUNCH("hm_pool_blocks");
     return HM_OK;
 }

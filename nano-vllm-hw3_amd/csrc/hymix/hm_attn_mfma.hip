@@ -15,7 +15,8 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const unsigned short* _
                                                          const int32_t* __restrict__ qstart, const int32_t* __restrict__ seq_pos0,
                                                          const float* __restrict__ sink, int window, int keep_first, float scale,
                                                          unsigned short* __restrict__ o, int H, int G, int D, int V, int block_size,
-                                                         int max_blocks) {
+                                                         int max_blocks, const unsigned short* __restrict__ kp,
+                                                         const unsigned short* __restrict__ vp, int pool, int pool_rows) {
     __shared__ __attribute__((aligned(16))) unsigned char lds_k[TileGeom<NBK>::LDS_BYTES];
     __shared__ __attribute__((aligned(16))) unsigned char lds_v[TileGeom<NBV>::LDS_BYTES];
     const int b = blockIdx.y, g = blockIdx.z, rep = H / G;
@@ -31,13 +32,13 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const unsigned short* _
     const int row_pos = pos0 + tok;
     const int wave_min_pos = pos0 + min(tile0 + 32 * wave, rows - 1) / rep;
     const int n_keys = pos0 + min(tile0 + 127, rows - 1) / rep + 1;
-    const TileWalk walk = make_walk(pos0 + tile0 / rep, window, keep_first);
+    const TileWalk walk = make_walk(pos0 + tile0 / rep, n_keys - 1, window, keep_first, pool);
     const float c_log2 = scale * 1.4426950408889634f;
     f32x16 oacc[NBV];
     float m_run, l_tot;
     kv_tile_loop<NBK, NBV, 4>(q + ((size_t)(q0 + tok) * H + head) * D, kc, vc, block_tables + (size_t)b * max_blocks, D, V, G, g,
                               block_size, walk, 0, walk.count(n_keys), n_keys, row_pos, wave_min_pos, window, keep_first, c_log2,
-                              lds_k, lds_v, oacc, m_run, l_tot);
+                              kp, vp, pool, pool_rows, lds_k, lds_v, oacc, m_run, l_tot);
     if (r >= rows) return;
     // the sink joins the denominator with its own score, which is not scaled (m_run is finite: a row sees itself)
     const float den = l_tot + (sink ? expf(sink[head] - m_run * scale) : 0.f);
@@ -63,12 +64,14 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(const unsigned short* _
                                                          const unsigned short* __restrict__ vc,
                                                          const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx,
                                                          int window, int keep_first, float scale, float* __restrict__ ws, int H,
-                                                         int G, int D, int V, int block_size, int max_blocks, int splits) {
+                                                         int G, int D, int V, int block_size, int max_blocks, int splits,
+                                                         const unsigned short* __restrict__ kp,
+                                                         const unsigned short* __restrict__ vp, int pool, int pool_rows) {
     __shared__ __attribute__((aligned(16))) unsigned char lds_k[TileGeom<NBK>::LDS_BYTES];
     __shared__ __attribute__((aligned(16))) unsigned char lds_v[TileGeom<NBV>::LDS_BYTES];
     const int sp = blockIdx.x, b = blockIdx.y, g = blockIdx.z, rep = H / G;
     const int n = ctx[b];
-    const TileWalk walk = make_walk(n - 1, window, keep_first);
+    const TileWalk walk = make_walk(n - 1, n - 1, window, keep_first, pool);
     const int nt = walk.count(n), per = (nt + splits - 1) / splits;
     const int vt_lo = sp * per, vt_hi = min(nt, vt_lo + per);
     const int lane = threadIdx.x & 63, l31 = lane & 31, hi = lane >> 5;
@@ -82,7 +85,8 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(const unsigned short* _
     f32x16 oacc[NBV];
     float m_run, l_tot;
     kv_tile_loop<NBK, NBV, 1>(q + ((size_t)b * H + head) * D, kc, vc, block_tables + (size_t)b * max_blocks, D, V, G, g, block_size,
-                              walk, vt_lo, vt_hi, n, n - 1, n - 1, window, keep_first, c_log2, lds_k, lds_v, oacc, m_run, l_tot);
+                              walk, vt_lo, vt_hi, n, n - 1, n - 1, window, keep_first, c_log2, kp, vp, pool, pool_rows, lds_k, lds_v,
+                              oacc, m_run, l_tot);
     if (l31 >= rep) return;
     if (hi == 0) { part[0] = l_tot > 0.f ? m_run * c_log2 : -INFINITY; part[1] = l_tot; }
 #pragma unroll
@@ -124,6 +128,11 @@ static int padded_nb(int n) {
     return nb <= 2 ? nb : 4;
 }
 
+static bool pool_args_ok(const void* kp, const void* vp, int pool, int pool_rows, int window, int keep_first, int block_size) {
+    if (pool < 0) return false;
+    return pool == 0 || (kp && vp && window > 0 && keep_first == 0 && pool_rows > 0 && (int64_t)pool_rows * pool >= block_size);
+}
+
 static bool shape_ok(int H, int G, int D, int V, int block_size) {
     return D % 8 == 0 && V % 8 == 0 && D <= 128 && V <= 128 && block_size % kTileKeys == 0 && H % G == 0;
 }
@@ -143,8 +152,9 @@ using namespace hm;
 extern "C" int hm_attn_tiles(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                              const int32_t* qstart, const int32_t* seq_pos0, const float* sink, int window, int keep_first,
                              float scale, void* o, int B, int max_q, int H, int G, int D, int V, int block_size, int max_blocks,
-                             void* stream) {
+                             const void* kp_cache, const void* vp_cache, int pool, int pool_rows, void* stream) {
     if (B < 0 || max_q < 0 || H < 1 || G < 1 || D < 1 || V < 1 || block_size < 1 || max_blocks < 1 || window < 0 || keep_first < 0 ||
+        !pool_args_ok(kp_cache, vp_cache, pool, pool_rows, window, keep_first, block_size) ||
         (B > 0 && max_q > 0 && (!q || !k_cache || !v_cache || !block_tables || !qstart || !seq_pos0 || !o))) {
         set_error("hm_attn_tiles: bad argument");
         return HM_EINVAL;
@@ -161,7 +171,8 @@ extern "C" int hm_attn_tiles(const void* q, const void* k_cache, const void* v_c
 #define HM_TILES(K_, V_)                                                                                                     \
     hipLaunchKernelGGL((attn_tiles_kernel<K_, V_>), grid, block, 0, s, (const unsigned short*)q, (const unsigned short*)k_cache, \
                        (const unsigned short*)v_cache, block_tables, qstart, seq_pos0, sink, window, keep_first, scale,       \
-                       (unsigned short*)o, H, G, D, V, block_size, max_blocks)
+                       (unsigned short*)o, H, G, D, V, block_size, max_blocks, (const unsigned short*)kp_cache,               \
+                       (const unsigned short*)vp_cache, pool, pool_rows)
     HM_BY_HEAD_SIZE(nbk, nbv, HM_TILES);
 #undef HM_TILES
     HM_CHECK_LAUNCH("hm_attn_tiles");
@@ -176,8 +187,10 @@ extern "C" size_t hm_attn_decode_workspace_bytes(int64_t B, int H, int V, int sp
 extern "C" int hm_attn_decode(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                               const int32_t* ctx, const float* sink, int window, int keep_first, float scale, void* o, int64_t B,
                               int H, int G, int D, int V, int block_size, int max_blocks, int splits, void* workspace,
-                              size_t workspace_bytes, void* stream) {
+                              size_t workspace_bytes, const void* kp_cache, const void* vp_cache, int pool, int pool_rows,
+                              void* stream) {
     if (B < 0 || H < 1 || G < 1 || D < 1 || V < 1 || block_size < 1 || max_blocks < 1 || splits < 1 || window < 0 || keep_first < 0 ||
+        !pool_args_ok(kp_cache, vp_cache, pool, pool_rows, window, keep_first, block_size) ||
         (B > 0 && (!q || !k_cache || !v_cache || !block_tables || !ctx || !o || !workspace))) {
         set_error("hm_attn_decode: bad argument");
         return HM_EINVAL;
@@ -197,7 +210,8 @@ extern "C" int hm_attn_decode(const void* q, const void* k_cache, const void* v_
 #define HM_DEC(K_, V_)                                                                                                        \
     hipLaunchKernelGGL((attn_decode_kernel<K_, V_>), grid, dim3(64), 0, s, (const unsigned short*)q, (const unsigned short*)k_cache, \
                        (const unsigned short*)v_cache, block_tables, ctx, window, keep_first, scale, (float*)workspace, H, G, D, \
-                       V, block_size, max_blocks, splits)
+                       V, block_size, max_blocks, splits, (const unsigned short*)kp_cache, (const unsigned short*)vp_cache, pool, \
+                       pool_rows)
     HM_BY_HEAD_SIZE(nbk, nbv, HM_DEC);
 #undef HM_DEC
     HM_CHECK_LAUNCH("hm_attn_decode");

@@ -12,7 +12,9 @@
 //
 // Tiles are 64 keys from key 0, whatever the step brings, so the order of every sum depends on positions alone.  With a
 // window the walk is over a list: the tiles that hold kept first tokens, then the tiles from the window's start; tiles
-// between are skipped (every score in them is masked, and a masked score adds an exact zero).
+// between are skipped (every score in them is masked, and a masked score adds an exact zero).  With pooled blocks the
+// list starts with tiles of 64 pooled entries (block means, read from the pooled caches row by row through the block
+// table); an entry is masked for the rows whose window has not yet passed its block.
 #pragma once
 #include "hm_common.h"
 
@@ -33,14 +35,22 @@ struct TileGeom {
 // The list of tiles a group of rows walks.  keep_tiles tiles from key 0, then tiles from key win_lo (a multiple of 64,
 // >= 64 keep_tiles) up to the causal end.
 struct TileWalk {
-    int keep_tiles, win_lo;
-    __device__ __forceinline__ int key0(int vt) const { return vt < keep_tiles ? vt * kTileKeys : win_lo + (vt - keep_tiles) * kTileKeys; }
-    __device__ __forceinline__ int count(int n_keys) const { return keep_tiles + (n_keys - win_lo + kTileKeys - 1) / kTileKeys; }
+    int pool_tiles, n_pool, keep_tiles, win_lo;
+    // first key of token tile vt (vt >= pool_tiles); a pooled tile vt < pool_tiles starts at entry 64 vt
+    __device__ __forceinline__ int key0(int vt) const {
+        const int u = vt - pool_tiles;
+        return u < keep_tiles ? u * kTileKeys : win_lo + (u - keep_tiles) * kTileKeys;
+    }
+    __device__ __forceinline__ int count(int n_keys) const {
+        return pool_tiles + keep_tiles + (n_keys - win_lo + kTileKeys - 1) / kTileKeys;
+    }
 };
 
-// min_pos = the smallest position among the rows that walk together, n_keys = 1 + the largest
-__device__ __forceinline__ TileWalk make_walk(int min_pos, int window, int keep_first) {
+// min_pos / max_pos = the smallest / largest position among the rows that walk together
+__device__ __forceinline__ TileWalk make_walk(int min_pos, int max_pos, int window, int keep_first, int pool) {
     TileWalk w;
+    w.n_pool = pooled_seen(max_pos, window, pool);
+    w.pool_tiles = (w.n_pool + kTileKeys - 1) / kTileKeys;
     if (window <= 0) { w.keep_tiles = 0; w.win_lo = 0; return w; }
     w.win_lo = max(0, min_pos - window + 1) / kTileKeys * kTileKeys;
     w.keep_tiles = min((keep_first + kTileKeys - 1) / kTileKeys, w.win_lo / kTileKeys);
@@ -56,7 +66,8 @@ __device__ __forceinline__ void kv_tile_loop(const unsigned short* __restrict__ 
                                              const unsigned short* __restrict__ vc, const int32_t* __restrict__ table, int D, int V,
                                              int G, int g, int block_size, TileWalk walk, int vt_lo, int vt_hi, int n_keys,
                                              int row_pos, int wave_min_pos, int window, int keep_first, float c_log2,
-                                             unsigned char* lds_k, unsigned char* lds_v, f32x16 (&oacc)[NBV], float& m_run,
+                                             const unsigned short* __restrict__ kp, const unsigned short* __restrict__ vp,
+                                             int pool, int pool_rows, unsigned char* lds_k, unsigned char* lds_v, f32x16 (&oacc)[NBV], float& m_run,
                                              float& l_tot) {
     typedef TileGeom<NBK> GK;
     typedef TileGeom<NBV> GV;
@@ -73,7 +84,31 @@ __device__ __forceinline__ void kv_tile_loop(const unsigned short* __restrict__ 
     }
 
     i32x4 kreg[NLK], vreg[NLV];
-    auto load_tile = [&](int kt0) {
+    auto load_tile = [&](int vt) {
+        if (vt < walk.pool_tiles) {                        // 64 pooled entries, each found through the block table
+#pragma unroll
+            for (int j = 0; j < NLK; ++j) {
+                const int c = tid + 64 * WAVES * j;
+                const int row = c / GK::CH, ch = c % GK::CH;
+                const int e = min(vt * kTileKeys + row, walk.n_pool - 1);
+                const size_t prow = (size_t)table[e / pool_rows] * pool_rows + e % pool_rows;
+                i32x4 v = {0, 0, 0, 0};
+                if (ch * 8 < D) v = *(const i32x4*)(kp + (prow * G + g) * D + ch * 8);
+                kreg[j] = v;
+            }
+#pragma unroll
+            for (int j = 0; j < NLV; ++j) {
+                const int c = tid + 64 * WAVES * j;
+                const int row = c / GV::CH, ch = c % GV::CH;
+                const int e = min(vt * kTileKeys + row, walk.n_pool - 1);
+                const size_t prow = (size_t)table[e / pool_rows] * pool_rows + e % pool_rows;
+                i32x4 v = {0, 0, 0, 0};
+                if (ch * 8 < V) v = *(const i32x4*)(vp + (prow * G + g) * V + ch * 8);
+                vreg[j] = v;
+            }
+            return;
+        }
+        const int kt0 = walk.key0(vt);
         const size_t row0 = (size_t)table[kt0 / block_size] * block_size + (kt0 % block_size);
 #pragma unroll
         for (int j = 0; j < NLK; ++j) {
@@ -115,15 +150,17 @@ __device__ __forceinline__ void kv_tile_loop(const unsigned short* __restrict__ 
     float l_run = 0.f;
     const int gq = (lane >> 4) & 1, ti = lane & 15, tq = ti >> 2, tp = ti & 3;      // transposed-read address pieces
 
-    load_tile(walk.key0(vt_lo));
+    const int my_pool = pooled_seen(row_pos, window, pool);   // pooled entries this row sees
+    load_tile(vt_lo);
     store_tile();
     __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < 2 * NBK; ++ks) asm volatile("" ::"v"(__builtin_bit_cast(i32x4, qf[ks])));   // loaded before the loop
     for (int vt = vt_lo; vt < vt_hi; ++vt) {
-        const int kt0 = walk.key0(vt);
+        const bool pooled = vt < walk.pool_tiles;
+        const int kt0 = pooled ? vt * kTileKeys : walk.key0(vt);
         const bool more = vt + 1 < vt_hi;
-        if (more) load_tile(walk.key0(vt + 1));
+        if (more) load_tile(vt + 1);
 
         f32x16 s[2];
 #pragma unroll
@@ -136,7 +173,15 @@ __device__ __forceinline__ void kv_tile_loop(const unsigned short* __restrict__ 
                 s[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[j], 0, 0, 0);
             }
         }
-        if (window > 0 || kt0 + kTileKeys - 1 > wave_min_pos) {
+        if (pooled) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int e = kt0 + 32 * j + (r & 3) + 8 * (r >> 2) + 4 * hi;
+                    if (e >= my_pool) s[j][r] = -INFINITY;
+                }
+        } else if (window > 0 || kt0 + kTileKeys - 1 > wave_min_pos) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll

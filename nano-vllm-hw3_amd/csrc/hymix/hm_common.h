@@ -38,6 +38,13 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 
 __device__ __forceinline__ float sigmoid_f(float v) { return 1.f / (1.f + expf(-v)); }
 
+// Pooled blocks a query at position `pos` sees beside its window: the blocks of `pool` tokens whose last token lies at
+// or before pos - window.  (Block e of a sequence is row e % pool_rows of the pooled page block_table[e / pool_rows];
+// pool_rows * pool >= block_size, so that page exists as soon as the block is complete.)
+__host__ __device__ __forceinline__ int pooled_seen(int pos, int window, int pool) {
+    return (pool > 0 && window > 0 && pos + 1 - window > 0) ? (pos + 1 - window) / pool : 0;
+}
+
 static inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
 
 #define HM_CHECK_LAUNCH(name)                                                    \

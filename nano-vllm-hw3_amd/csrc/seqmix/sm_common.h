@@ -43,6 +43,14 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     return t;
 }
 
+// what an expert applies between its two products (SM_ACT_*): the clamped GLU of a gate and an up product, or a GELU
+// of the up product alone (exact, or the tanh form)
+__device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752f)); }
+__device__ __forceinline__ float gelu_tanh(float z) {
+    return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ float plain_act(float z, int act) { return act == SM_ACT_GELU_TANH ? gelu_tanh(z) : gelu_erf(z); }
+
 static inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
 
 #define SM_CHECK_LAUNCH(name)                                                    \

@@ -30,12 +30,14 @@ struct TileGeom {
 // row_pos; wave_min_pos = the smallest row_pos of the wave (tiles wholly below it skip the mask).  Every wave of the
 // workgroup must call this with the same key range.  On return oacc holds the unnormalised output (lane: query
 // l & 31, columns 32 d + 8 (r >> 2) + 4 (l >> 5) + (r & 3)), m_run the row maximum of the raw scores and l_tot the
-// sum of exp2((s - m_run) * c_log2) over the row.
-template <int NB, int WAVES>
+// sum of exp2((s - m_run) * c_log2) over the row.  Only the first 32 NBV columns of a cache row are values (NBV <= NB:
+// the rest of the row is key only, e.g. a rotated part).  window > 0: a row sees only the keys > row_pos - window; a
+// row whose window starts behind the range's first tiles has seen nothing there (its maximum stays -inf, its weights 0).
+template <int NB, int NBV, int WAVES>
 __device__ __forceinline__ void latent_tile_loop(const unsigned short* __restrict__ qrow, const unsigned short* __restrict__ cache,
                                                  const int32_t* __restrict__ table, int R, int block_size, int k_lo, int k_hi,
-                                                 int row_pos, int wave_min_pos, float c_log2, unsigned char* lds,
-                                                 f32x16 (&oacc)[NB], float& m_run, float& l_tot) {
+                                                 int row_pos, int wave_min_pos, float c_log2, int window, unsigned char* lds,
+                                                 f32x16 (&oacc)[NBV], float& m_run, float& l_tot) {
     typedef TileGeom<NB> G;
     constexpr int NLD = G::CH / WAVES;                     // 16-byte chunks a thread stages per tile
     const int tid = threadIdx.x, lane = tid & 63, l31 = lane & 31, hi = lane >> 5;
@@ -71,7 +73,7 @@ __device__ __forceinline__ void latent_tile_loop(const unsigned short* __restric
     };
 
 #pragma unroll
-    for (int d = 0; d < NB; ++d)
+    for (int d = 0; d < NBV; ++d)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[d][r] = 0.f;
     m_run = -INFINITY;
@@ -98,13 +100,13 @@ __device__ __forceinline__ void latent_tile_loop(const unsigned short* __restric
                 s[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cf, qf[ks], s[j], 0, 0, 0);
             }
         }
-        if (kt0 + kTileKeys - 1 > wave_min_pos) {
+        if (window > 0 || kt0 + kTileKeys - 1 > wave_min_pos) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = kt0 + 32 * j + (r & 3) + 8 * (r >> 2) + 4 * hi;
-                    if (key > row_pos) s[j][r] = -INFINITY;
+                    if (key > row_pos || (window > 0 && row_pos - key >= window)) s[j][r] = -INFINITY;
                 }
         }
         float mx = s[0][0];
@@ -113,9 +115,11 @@ __device__ __forceinline__ void latent_tile_loop(const unsigned short* __restric
 #pragma unroll
             for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[j][r]);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);              // finite: the first key of the range is visible to every row
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c_log2);
-        const float mc = m_new * c_log2;
+        const float m_new = fmaxf(m_run, mx);
+        // without a window the first key of the range is visible to every row; with one a row may have seen nothing yet
+        const bool none = m_new == -INFINITY;
+        const float alpha = none ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new) * c_log2);
+        const float mc = none ? 0.f : m_new * c_log2;
         float psum = 0.f;
         bf16x8 pf[2][2];
 #pragma unroll
@@ -132,12 +136,12 @@ __device__ __forceinline__ void latent_tile_loop(const unsigned short* __restric
         m_run = m_new;
         if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
-            for (int d = 0; d < NB; ++d)
+            for (int d = 0; d < NBV; ++d)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) oacc[d][r] *= alpha;
         }
 #pragma unroll
-        for (int d = 0; d < NB; ++d)
+        for (int d = 0; d < NBV; ++d)
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -162,3 +166,19 @@ __device__ __forceinline__ void latent_tile_loop(const unsigned short* __restric
 }
 
 }  // namespace sm
+
+// run M(NB, NBV) with the padded key and value widths of a latent row: rows whose values are the whole row, and the
+// common case of a rotated key part of up to 64 columns behind the values
+#define SM_BY_LATENT_SIZE(nb, nbv, M)                                                         \
+    do {                                                                                      \
+        if (nbv == nb || nb - nbv > 2) {                                                      \
+            if (nb <= 1) M(1, 1); else if (nb == 2) M(2, 2); else if (nb == 3) M(3, 3);       \
+            else if (nb == 4) M(4, 4); else if (nb <= 6) M(6, 6); else M(8, 8);               \
+        } else if (nb - nbv == 1) {                                                           \
+            if (nb == 2) M(2, 1); else if (nb == 3) M(3, 2); else if (nb == 4) M(4, 3);       \
+            else if (nb == 5) M(5, 4); else if (nb <= 7) M(7, 6); else M(8, 7);               \
+        } else {                                                                              \
+            if (nb == 3) M(3, 1); else if (nb == 4) M(4, 2); else if (nb <= 6) M(6, 4);       \
+            else M(8, 6);                                                                     \
+        }                                                                                     \
+    } while (0)

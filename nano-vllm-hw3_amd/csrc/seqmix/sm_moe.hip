@@ -1,4 +1,5 @@
-// Mixture of experts: the router (softmax scores, group-limited top-k, renormalised weights) and the expert products
+// Mixture of experts: the router (softmax or sigmoid scores, an optional correction that only steers the choice,
+// group-limited top-k, weights renormalised or not) and the expert products
 // in their memory-bound form, one (token, chosen expert) pair at a time.
 #include "sm_common.h"
 
@@ -11,7 +12,8 @@ constexpr int kRouteTokens = 8;      // tokens per workgroup: every router row r
 template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router_w,
                                                         int32_t* __restrict__ idx, float* __restrict__ wts, int64_t T_all, int W,
-                                                        int E, int top, int groups, int keep) {
+                                                        int E, int top, int groups, int keep, int score,
+                                                        const float* __restrict__ correction, int group_top, int renorm) {
     extern __shared__ float z_all[];             // per token: E scores, then `groups` group scores
     const int64_t t0 = (int64_t)blockIdx.x * kRouteTokens;
     const int nt = (int)min((int64_t)kRouteTokens, T_all - t0);
@@ -35,13 +37,72 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     // one thread finishes a token: E is small and the selections are sequential by nature
     const int64_t t = t0 + threadIdx.x;
     float* z = z_all + threadIdx.x * (E + groups);
-    float mx = -INFINITY;
-    for (int e = 0; e < E; ++e) mx = fmaxf(mx, z[e]);
-    float sum = 0.f;
-    for (int e = 0; e < E; ++e) { z[e] = expf(z[e] - mx); sum += z[e]; }
-    const float inv = 1.f / sum;
-    for (int e = 0; e < E; ++e) z[e] *= inv;
+    if (score == SM_ROUTE_SIGMOID) {
+        for (int e = 0; e < E; ++e) z[e] = 1.f / (1.f + expf(-z[e]));
+    } else {
+        float mx = -INFINITY;
+        for (int e = 0; e < E; ++e) mx = fmaxf(mx, z[e]);
+        float sum = 0.f;
+        for (int e = 0; e < E; ++e) { z[e] = expf(z[e] - mx); sum += z[e]; }
+        const float inv = 1.f / sum;
+        for (int e = 0; e < E; ++e) z[e] *= inv;
+    }
     float* gs = z + E;
+    if (correction != nullptr || group_top > 1) {
+        // The general form: choice scores c = s + correction (they may be negative) decide, the weights are s.  A group
+        // scores the sum of its `group_top` largest c; experts outside the best `keep` groups count as -inf.
+        const int per = E / groups;
+        bool ok_all = groups <= 1;
+        if (!ok_all) {
+            for (int g = 0; g < groups; ++g) {
+                float tot = 0.f;
+                int used[4] = {-1, -1, -1, -1};                 // group_top <= 4
+                for (int k = 0; k < group_top && k < per; ++k) {
+                    int best = -1;
+                    float bv = -INFINITY;
+                    for (int e = 0; e < per; ++e) {
+                        bool taken = false;
+                        for (int j = 0; j < k; ++j) taken |= used[j] == e;
+                        const float c = z[g * per + e] + (correction ? correction[g * per + e] : 0.f);
+                        if (!taken && (best < 0 || c > bv)) { bv = c; best = e; }
+                    }
+                    used[k] = best;
+                    tot += bv;
+                }
+                gs[g] = tot;
+            }
+            // keep the best groups: a kept group's score becomes +inf, the others' -inf afterwards
+            for (int k = 0; k < keep; ++k) {
+                int best = -1;
+                float bv = -INFINITY;
+                for (int g = 0; g < groups; ++g)
+                    if (gs[g] != INFINITY && (best < 0 || gs[g] > bv)) { bv = gs[g]; best = g; }
+                if (best >= 0) gs[best] = INFINITY;
+            }
+        }
+        int chosen[kMaxTop];
+        float cw[kMaxTop], tot = 0.f;
+        for (int k = 0; k < top; ++k) {
+            int best = -1;
+            float bv = -INFINITY;
+            for (int e = 0; e < E; ++e) {
+                if (!ok_all && gs[e / per] != INFINITY) continue;
+                bool taken = false;
+                for (int j = 0; j < k; ++j) taken |= chosen[j] == e;
+                const float c = z[e] + (correction ? correction[e] : 0.f);
+                if (!taken && (best < 0 || c > bv)) { bv = c; best = e; }
+            }
+            chosen[k] = best < 0 ? 0 : best;
+            cw[k] = best < 0 ? 0.f : z[best];
+            tot += cw[k];
+        }
+        const float rn = renorm ? 1.f / (tot + 1e-20f) : 1.f;
+        for (int k = 0; k < top; ++k) {
+            idx[(size_t)t * top + k] = chosen[k];
+            wts[(size_t)t * top + k] = cw[k] * rn;
+        }
+        return;
+    }
     if (groups > 1) {
         const int per = E / groups;
         for (int g = 0; g < groups; ++g) {
@@ -74,7 +135,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
         cw[k] = best < 0 ? 0.f : bv;
         tot += cw[k];
     }
-    const float rn = 1.f / (tot + 1e-20f);
+    const float rn = renorm ? 1.f / (tot + 1e-20f) : 1.f;
     for (int k = 0; k < top; ++k) {
         idx[(size_t)t * top + k] = chosen[k];
         wts[(size_t)t * top + k] = cw[k] * rn;
@@ -91,13 +152,24 @@ __device__ __forceinline__ float clamped_glu(float g, float u, float limit, floa
 template <typename T>
 __global__ __launch_bounds__(256) void moe_pairs_gate_up_kernel(const T* __restrict__ h, const int32_t* __restrict__ idx,
                                                                 const T* __restrict__ w_gu, float limit, float alpha,
-                                                                T* __restrict__ act, int top, int W, int F) {
+                                                                T* __restrict__ act, int top, int W, int F, int act_kind) {
     extern __shared__ float h_lds[];
     const int64_t p = blockIdx.x, t = p / top;
     const int e = idx[p];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int c = threadIdx.x; c < W; c += 256) h_lds[c] = to_f(h[(size_t)t * W + c]);
     __syncthreads();
+    if (act_kind != SM_ACT_CLAMPED_GLU) {            // one product per expert: w_gu is [E, F, W]
+        const T* wu = w_gu + (size_t)e * F * W;
+        for (int f = wave; f < F; f += 4) {
+            const T* u_row = wu + (size_t)f * W;
+            float u = 0.f;
+            for (int c = lane; c < W; c += 64) u += h_lds[c] * to_f(u_row[c]);
+            u = wave_sum(u);
+            if (lane == 0) act[(size_t)p * F + f] = from_f<T>(plain_act(to_f(from_f<T>(u)), act_kind));
+        }
+        return;
+    }
     const T* wg = w_gu + (size_t)e * 2 * F * W;
     for (int f = wave; f < F; f += 4) {
         const T* g_row = wg + (size_t)f * W;
@@ -147,8 +219,10 @@ __global__ __launch_bounds__(256) void moe_pairs_down_kernel(const T* __restrict
 using namespace sm;
 
 extern "C" int sm_moe_route(int dtype, const void* h, const float* router_w, int32_t* idx, float* wts, int64_t T, int W, int E,
-                            int top, int groups, int keep, void* stream) {
-    if (T < 0 || W < 1 || E < 1 || top < 1 || (T > 0 && (!h || !router_w || !idx || !wts))) {
+                            int top, int groups, int keep, int score, const float* correction, int group_top, int renorm,
+                            void* stream) {
+    if (T < 0 || W < 1 || E < 1 || top < 1 || (score != SM_ROUTE_SOFTMAX && score != SM_ROUTE_SIGMOID) || group_top < 1 ||
+        group_top > 4 || (T > 0 && (!h || !router_w || !idx || !wts))) {
         set_error("sm_moe_route: bad argument");
         return SM_EINVAL;
     }
@@ -161,14 +235,14 @@ extern "C" int sm_moe_route(int dtype, const void* h, const float* router_w, int
     SM_DISPATCH(dtype, "sm_moe_route",
                 hipLaunchKernelGGL(moe_route_kernel<DT>, dim3((unsigned)((T + kRouteTokens - 1) / kRouteTokens)), dim3(256),
                                    (size_t)kRouteTokens * (E + groups) * 4, as_stream(stream), (const DT*)h, router_w, idx, wts, T, W, E,
-                                   top, groups, keep));
+                                   top, groups, keep, score, correction, group_top, renorm));
     SM_CHECK_LAUNCH("sm_moe_route");
     return SM_OK;
 }
 
 extern "C" int sm_moe_pairs_gate_up(int dtype, const void* h, const int32_t* idx, const void* w_gu, float limit, float alpha,
-                                    void* act, int64_t T, int top, int W, int F, void* stream) {
-    if (T < 0 || top < 1 || W < 1 || F < 1 || (T > 0 && (!h || !idx || !w_gu || !act))) {
+                                    int act_kind, void* act, int64_t T, int top, int W, int F, void* stream) {
+    if (T < 0 || top < 1 || W < 1 || F < 1 || act_kind < 0 || act_kind > SM_ACT_GELU_TANH || (T > 0 && (!h || !idx || !w_gu || !act))) {
         set_error("sm_moe_pairs_gate_up: bad argument");
         return SM_EINVAL;
     }
@@ -176,7 +250,7 @@ extern "C" int sm_moe_pairs_gate_up(int dtype, const void* h, const int32_t* idx
     if (T == 0) return SM_OK;
     SM_DISPATCH(dtype, "sm_moe_pairs_gate_up",
                 hipLaunchKernelGGL(moe_pairs_gate_up_kernel<DT>, dim3((unsigned)(T * top)), dim3(256), (size_t)W * 4,
-                                   as_stream(stream), (const DT*)h, idx, (const DT*)w_gu, limit, alpha, (DT*)act, top, W, F));
+                                   as_stream(stream), (const DT*)h, idx, (const DT*)w_gu, limit, alpha, (DT*)act, top, W, F, act_kind));
     SM_CHECK_LAUNCH("sm_moe_pairs_gate_up");
     return SM_OK;
 }

@@ -62,11 +62,13 @@ __device__ __forceinline__ bf16x8 load8(const unsigned short* p, int k, int K) {
 
 // GATE_UP: A = h rows gathered by token, B = the expert's gate and up rows, out = act [rows, N] (N = F, K = W)
 // else:    A = act rows,                 B = the expert's down rows,       out = per-row products [rows, N] (N = W, K = F)
-template <bool GATE_UP>
+// MODE 0: the down product; 1: gate and up with the clamped GLU; 2: the up product alone with a GELU (act_kind)
+template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(const unsigned short* __restrict__ a, const unsigned short* __restrict__ w,
                                                           const int32_t* __restrict__ row_pair, const int32_t* __restrict__ tile_expert,
                                                           unsigned short* __restrict__ out, int top, int N, int K, float limit,
-                                                          float alpha) {
+                                                          float alpha, int act_kind) {
+    constexpr bool GATE_UP = MODE == 1, FROM_TOKENS = MODE != 0;
     const int tile = blockIdx.x;
     const int e = tile_expert[tile];
     if (e < 0) return;
@@ -76,7 +78,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const unsigned short* 
     if (n0 >= N) return;
     const int row = tile * kRowsPerTile + l31;
     const int pair = row_pair[row];
-    const unsigned short* ap = GATE_UP ? a + (size_t)(pair < 0 ? 0 : pair / top) * K : a + (size_t)row * K;
+    const unsigned short* ap = FROM_TOKENS ? a + (size_t)(pair < 0 ? 0 : pair / top) * K : a + (size_t)row * K;
     // weights in the tiled layout of sm_moe_tile_weights: block (expert, 32-row block, 64-k step) = 4 KB, chunk s of
     // lane L at 16 (64 s + L): a wave's load is one contiguous KB
     const int nb32 = (N + 31) / 32, ksteps = (K + 63) / 64;
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const unsigned short* 
     for (int r = 0; r < 16; ++r) {
         const int orow = tile * kRowsPerTile + (r & 3) + 8 * (r >> 2) + 4 * hi;
         if (row_pair[orow] < 0) continue;
-        const float v = GATE_UP ? glu_bf16(acc[r], acc2[r], limit, alpha) : acc[r];
+        const float v = GATE_UP ? glu_bf16(acc[r], acc2[r], limit, alpha) : (MODE == 2 ? plain_act((float)(bf16_t)acc[r], act_kind) : acc[r]);
         out[(size_t)orow * N + n0 + l31] = __builtin_bit_cast(unsigned short, (bf16_t)v);
     }
 }
@@ -152,9 +154,9 @@ extern "C" int sm_moe_grouped_tiles(int64_t T, int top, int E) {
 }
 
 extern "C" int sm_moe_grouped(const void* h, const int32_t* idx, const float* wts, const void* w_gu, const void* w_down,
-                              const void* shared, float limit, float alpha, void* y, int64_t T, int top, int E, int W, int F,
+                              const void* shared, float limit, float alpha, int act_kind, void* y, int64_t T, int top, int E, int W, int F,
                               int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row, void* act, void* prod, void* stream) {
-    if (T < 0 || top < 1 || E < 1 || W < 1 || F < 1 ||
+    if (T < 0 || top < 1 || E < 1 || W < 1 || F < 1 || act_kind < 0 || act_kind > SM_ACT_GELU_TANH ||
         (T > 0 && (!h || !idx || !wts || !w_gu || !w_down || !y || !row_pair || !tile_expert || !pair_row || !act || !prod))) {
         set_error("sm_moe_grouped: bad argument");
         return SM_EINVAL;
@@ -169,13 +171,18 @@ extern "C" int sm_moe_grouped(const void* h, const int32_t* idx, const float* wt
     hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)3 * E * sizeof(int), s, idx, (int)(T * top), E, tiles, row_pair,
                        tile_expert, pair_row);
     SM_CHECK_LAUNCH("sm_moe_grouped (align)");
-    hipLaunchKernelGGL(moe_grouped_kernel<true>, dim3((unsigned)tiles, (unsigned)((F + 127) / 128)), dim3(256), 0, s,
-                       (const unsigned short*)h, (const unsigned short*)w_gu, row_pair, tile_expert, (unsigned short*)act, top, F, W,
-                       limit, alpha);
+    if (act_kind == SM_ACT_CLAMPED_GLU)
+        hipLaunchKernelGGL(moe_grouped_kernel<1>, dim3((unsigned)tiles, (unsigned)((F + 127) / 128)), dim3(256), 0, s,
+                           (const unsigned short*)h, (const unsigned short*)w_gu, row_pair, tile_expert, (unsigned short*)act, top, F,
+                           W, limit, alpha, act_kind);
+    else
+        hipLaunchKernelGGL(moe_grouped_kernel<2>, dim3((unsigned)tiles, (unsigned)((F + 127) / 128)), dim3(256), 0, s,
+                           (const unsigned short*)h, (const unsigned short*)w_gu, row_pair, tile_expert, (unsigned short*)act, top, F,
+                           W, limit, alpha, act_kind);
     SM_CHECK_LAUNCH("sm_moe_grouped (gate/up)");
-    hipLaunchKernelGGL(moe_grouped_kernel<false>, dim3((unsigned)tiles, (unsigned)((W + 127) / 128)), dim3(256), 0, s,
+    hipLaunchKernelGGL(moe_grouped_kernel<0>, dim3((unsigned)tiles, (unsigned)((W + 127) / 128)), dim3(256), 0, s,
                        (const unsigned short*)act, (const unsigned short*)w_down, row_pair, tile_expert, (unsigned short*)prod, top, W,
-                       F, 0.f, 0.f);
+                       F, 0.f, 0.f, 0);
     SM_CHECK_LAUNCH("sm_moe_grouped (down)");
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)T), dim3(256), 0, s, (const unsigned short*)prod, pair_row, wts,
                        (const unsigned short*)shared, (unsigned short*)y, top, W);

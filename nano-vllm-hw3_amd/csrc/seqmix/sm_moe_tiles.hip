@@ -65,12 +65,14 @@ __device__ __forceinline__ i32x4 load16(const unsigned short* p, int k, int K) {
 
 // GATE_UP: A = h rows gathered by token, B = the expert's gate and up rows, out = act [rows, N] (N = F, K = W)
 // else:    A = act rows,                 B = the expert's down rows,       out = per-row products [rows, N] (N = W, K = F)
-template <bool GATE_UP>
+// MODE 0: the down product; 1: gate and up with the clamped GLU; 2: the up product alone with a GELU (act_kind)
+template <int MODE>
 __global__ __launch_bounds__(256) void moe_tiles128_kernel(const unsigned short* __restrict__ a, const unsigned short* __restrict__ w,
                                                            const int32_t* __restrict__ row_pair, const int32_t* __restrict__ tile_expert,
                                                            unsigned short* __restrict__ out, int top, int N, int K, float limit,
-                                                           float alpha) {
+                                                           float alpha, int act_kind) {
     __shared__ __attribute__((aligned(16))) unsigned char a_lds[kBigRows * kAStride];
+    constexpr bool GATE_UP = MODE == 1, FROM_TOKENS = MODE != 0;
     const int tile = blockIdx.x;
     const int e = tile_expert[tile];
     if (e < 0) return;                                        // (uniform over the workgroup)
@@ -80,7 +82,7 @@ __global__ __launch_bounds__(256) void moe_tiles128_kernel(const unsigned short*
     // staging: thread -> row tid / 2, k half tid % 2 (32 consecutive k = 64 bytes)
     const int srow = tid >> 1, shalf = tid & 1;
     const int spair = row_pair[tile * kBigRows + srow];
-    const unsigned short* ap = GATE_UP ? a + (size_t)(spair < 0 ? 0 : spair / top) * K : a + ((size_t)tile * kBigRows + srow) * K;
+    const unsigned short* ap = FROM_TOKENS ? a + (size_t)(spair < 0 ? 0 : spair / top) * K : a + ((size_t)tile * kBigRows + srow) * K;
     // weights in the tiled layout of sm_moe_tile_weights (see sm_moe_grouped.hip): a wave's load is one contiguous KB
     const int nb32 = (N + 31) / 32, ksteps = (K + 63) / 64;
     const unsigned short* bp = w + (((size_t)e * (GATE_UP ? 2 : 1) * nb32 + min(n0, N - 1) / 32) * ksteps) * 2048 + 8 * lane;
@@ -132,7 +134,8 @@ __global__ __launch_bounds__(256) void moe_tiles128_kernel(const unsigned short*
         for (int r = 0; r < 16; ++r) {
             const int orow = tile * kBigRows + 32 * m + (r & 3) + 8 * (r >> 2) + 4 * hi;
             if (row_pair[orow] < 0) continue;
-            const float v = GATE_UP ? glu_bf16_big(acc[m][r], acc2[m][r], limit, alpha) : acc[m][r];
+            const float v = GATE_UP ? glu_bf16_big(acc[m][r], acc2[m][r], limit, alpha)
+                                    : (MODE == 2 ? plain_act((float)(bf16_t)acc[m][r], act_kind) : acc[m][r]);
             out[(size_t)orow * N + n0 + l31] = __builtin_bit_cast(unsigned short, (bf16_t)v);
         }
 }
@@ -147,9 +150,9 @@ extern "C" int sm_moe_tiles128_count(int64_t T, int top, int E) {
 }
 
 extern "C" int sm_moe_tiles128(const void* h, const int32_t* idx, const float* wts, const void* w_gu, const void* w_down,
-                               const void* shared, float limit, float alpha, void* y, int64_t T, int top, int E, int W, int F,
+                               const void* shared, float limit, float alpha, int act_kind, void* y, int64_t T, int top, int E, int W, int F,
                                int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row, void* act, void* prod, void* stream) {
-    if (T < 0 || top < 1 || E < 1 || W < 1 || F < 1 ||
+    if (T < 0 || top < 1 || E < 1 || W < 1 || F < 1 || act_kind < 0 || act_kind > SM_ACT_GELU_TANH ||
         (T > 0 && (!h || !idx || !wts || !w_gu || !w_down || !y || !row_pair || !tile_expert || !pair_row || !act || !prod))) {
         set_error("sm_moe_tiles128: bad argument");
         return SM_EINVAL;
@@ -164,13 +167,18 @@ extern "C" int sm_moe_tiles128(const void* h, const int32_t* idx, const float* w
     hipLaunchKernelGGL(moe_align128_kernel, dim3(1), dim3(1024), (size_t)3 * E * sizeof(int), s, idx, (int)(T * top), E, tiles, row_pair,
                        tile_expert, pair_row);
     SM_CHECK_LAUNCH("sm_moe_tiles128 (align)");
-    hipLaunchKernelGGL(moe_tiles128_kernel<true>, dim3((unsigned)tiles, (unsigned)((F + 127) / 128)), dim3(256), 0, s,
-                       (const unsigned short*)h, (const unsigned short*)w_gu, row_pair, tile_expert, (unsigned short*)act, top, F, W,
-                       limit, alpha);
+    if (act_kind == SM_ACT_CLAMPED_GLU)
+        hipLaunchKernelGGL(moe_tiles128_kernel<1>, dim3((unsigned)tiles, (unsigned)((F + 127) / 128)), dim3(256), 0, s,
+                           (const unsigned short*)h, (const unsigned short*)w_gu, row_pair, tile_expert, (unsigned short*)act, top, F,
+                           W, limit, alpha, act_kind);
+    else
+        hipLaunchKernelGGL(moe_tiles128_kernel<2>, dim3((unsigned)tiles, (unsigned)((F + 127) / 128)), dim3(256), 0, s,
+                           (const unsigned short*)h, (const unsigned short*)w_gu, row_pair, tile_expert, (unsigned short*)act, top, F,
+                           W, limit, alpha, act_kind);
     SM_CHECK_LAUNCH("sm_moe_tiles128 (gate/up)");
-    hipLaunchKernelGGL(moe_tiles128_kernel<false>, dim3((unsigned)tiles, (unsigned)((W + 127) / 128)), dim3(256), 0, s,
+    hipLaunchKernelGGL(moe_tiles128_kernel<0>, dim3((unsigned)tiles, (unsigned)((W + 127) / 128)), dim3(256), 0, s,
                        (const unsigned short*)act, (const unsigned short*)w_down, row_pair, tile_expert, (unsigned short*)prod, top, W,
-                       F, 0.f, 0.f);
+                       F, 0.f, 0.f, 0);
     SM_CHECK_LAUNCH("sm_moe_tiles128 (down)");
     return sm_moe_combine(prod, pair_row, wts, shared, y, T, top, W, stream);
 }

@@ -23,21 +23,23 @@ SIGNATURES = {
     "sm_canon_conv": (_int, [_int, _vp, _vp, _vp, _int, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "sm_canon_update": (_int, [_int, _vp, _vp, _int, _int, _vp, _vp, _int, _int, _int, _vp]),
     "sm_latent_norm_store": (_int, [_int, _vp, _i64, _vp, _f, _vp, _vp, _i64, _int, _vp]),
-    "sm_latent_attn_rows": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i64, _int, _int, _int, _int, _vp]),
-    "sm_latent_attn_tiles": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _int, _int, _int, _int, _int, _int, _vp]),
+    "sm_latent_attn_rows": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i64, _int, _int, _int, _int, _int, _int, _vp]),
+    "sm_latent_rope_store": (_int, [_int, _vp, _i64, _vp, _f, _vp, _i64, _vp, _vp, _int, _vp, _vp, _vp, _i64, _int, _int, _int,
+                                    _int, _vp]),
+    "sm_latent_attn_tiles": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _int, _int, _int, _int, _int, _int, _int, _int, _vp]),
     "sm_latent_decode_workspace_bytes": (_sz, [_i64, _int, _int, _int]),
-    "sm_latent_attn_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _f, _i64, _int, _int, _int, _int, _int, _vp, _sz, _vp]),
+    "sm_latent_attn_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _f, _i64, _int, _int, _int, _int, _int, _vp, _sz, _int, _int, _vp]),
     "sm_poly_norm": (_int, [_int, _vp, _vp, _f, _vp, _i64, _int, _vp]),
     "sm_clamped_glu": (_int, [_int, _vp, _f, _f, _vp, _i64, _int, _vp]),
-    "sm_moe_route": (_int, [_int, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _int, _int, _vp]),
-    "sm_moe_pairs_gate_up": (_int, [_int, _vp, _vp, _vp, _f, _f, _vp, _i64, _int, _int, _int, _vp]),
+    "sm_moe_route": (_int, [_int, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _int, _int, _int, _vp, _int, _int, _vp]),
+    "sm_moe_pairs_gate_up": (_int, [_int, _vp, _vp, _vp, _f, _f, _int, _vp, _i64, _int, _int, _int, _vp]),
     "sm_moe_pairs_down": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _vp]),
     "sm_moe_grouped_tiles": (_int, [_i64, _int, _int]),
     "sm_moe_tiles128_count": (_int, [_i64, _int, _int]),
-    "sm_moe_tiles128": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "sm_moe_tiles128": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _int, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp]),
     "sm_moe_align": (_int, [_vp, _i64, _int, _int, _vp, _vp, _vp, _vp]),
     "sm_moe_combine": (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
-    "sm_moe_grouped": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "sm_moe_grouped": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _f, _f, _int, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp]),
 }
 
 _lib = None

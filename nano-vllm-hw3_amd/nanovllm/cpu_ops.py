@@ -131,8 +131,35 @@ def latent_norm_store(x, w, eps, cache, slot_mapping):
     cache.view(-1, cache.shape[-1])[slot_mapping[keep].long()] = c[keep]
 
 
-def latent_attention(q, cache, ctx, scale):
-    o = torch.empty_like(q)
+def rotate_pairs(x, pos, inv_freq, rot_dims):
+    """Channels (2i, 2i + 1), i < rot_dims / 2, of the last dimension turned by pos * inv_freq[i]; x [T, ..., C] f32."""
+    if not rot_dims:
+        return x
+    ang = pos.float()[:, None] * inv_freq.float()[None, :]
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [rot_dims // 2]
+    c, s = torch.cos(ang).view(shape), torch.sin(ang).view(shape)
+    u, v = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+    out = x.clone()
+    out[..., 0:rot_dims:2] = u * c - v * s
+    out[..., 1:rot_dims:2] = v * c + u * s
+    return out
+
+
+def latent_rope_store(x, w, eps, q, qa, inv_freq, rot_dims, H, D, R, Rd, cache, ctx):
+    T = x.shape[0]
+    xf = x.float()
+    c = xf[:, :R] * torch.rsqrt(xf[:, :R].pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    kr = rotate_pairs(xf[:, R:], ctx.tok_pos, inv_freq, rot_dims)
+    rows = ctx.slot_mapping
+    keep = rows >= 0
+    cache.view(-1, R + Rd)[rows[keep].long()] = torch.cat([c, kr], -1).to(cache.dtype)[keep]
+    qr = rotate_pairs(q.float().view(T, H, D + Rd)[..., D:], ctx.tok_pos, inv_freq, rot_dims)
+    qa[..., R:] = qr.to(qa.dtype)
+
+
+def latent_attention(q, cache, ctx, scale, RV=0, window=0):
+    RV = RV or q.shape[-1]
+    o = torch.empty(q.shape[:-1] + (RV,), dtype=q.dtype)
     bs = cache.shape[1]
     rows = cache.view(-1, cache.shape[-1])
     qs = ctx.qstart.tolist()
@@ -145,8 +172,11 @@ def latent_attention(q, cache, ctx, scale):
         c = rows[ctx.block_tables[b, t // bs].long() * bs + t % bs].float()          # [n, R]
         s = torch.einsum("thr,nr->thn", q[a:e].float(), c) * scale
         pos = ctx.tok_pos[a:e].long()
-        s = s.masked_fill(t[None, None, :] > pos[:, None, None], float("-inf"))
-        o[a:e] = torch.einsum("thn,nr->thr", torch.softmax(s, -1), c).to(q.dtype)
+        hidden = t[None, None, :] > pos[:, None, None]
+        if window > 0:
+            hidden = hidden | (pos[:, None, None] - t[None, None, :] >= window)
+        s = s.masked_fill(hidden, float("-inf"))
+        o[a:e] = torch.einsum("thn,nr->thr", torch.softmax(s, -1), c[:, :RV]).to(q.dtype)
     return o
 
 
@@ -166,25 +196,30 @@ def clamped_glu(gu, limit, alpha):
     return (g * torch.sigmoid(alpha * g) * (u + 1)).to(gu.dtype)
 
 
-def moe_route(h, router_w, top, groups, keep):
+def moe_route(h, router_w, top, groups, keep, score=0, correction=None, group_top=1, renorm=True):
     T, E = h.shape[0], router_w.shape[0]
-    s = torch.softmax(h.float() @ router_w.t(), -1)
-    masked = s
+    z = h.float() @ router_w.t()
+    s = torch.sigmoid(z) if score == 1 else torch.softmax(z, -1)
+    choice = s if correction is None else s + correction.float()
+    masked = choice
     if groups > 1:
         per = E // groups
-        best = s.view(T, groups, per).amax(-1).topk(keep, -1).indices
+        best = choice.view(T, groups, per).topk(min(group_top, per), -1).values.sum(-1).topk(keep, -1).indices
         ok = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, best, True)
-        masked = s.masked_fill(~ok.repeat_interleave(per, 1), -1.0)
+        masked = choice.masked_fill(~ok.repeat_interleave(per, 1), float("-inf"))
     idx = masked.topk(top, -1).indices
     w = s.gather(1, idx)
-    return idx.int(), w / (w.sum(-1, keepdim=True) + 1e-20)
+    return idx.int(), (w / (w.sum(-1, keepdim=True) + 1e-20) if renorm else w)
 
 
-def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared):
+def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared, act_kind=0):
     y = torch.zeros(h.shape, dtype=torch.float32)
     for e in idx.unique().tolist():
         tok, k = (idx == e).nonzero(as_tuple=True)
-        act = clamped_glu(F.linear(h[tok], w_gu[e]), limit, alpha)
+        if act_kind == 0:
+            act = clamped_glu(F.linear(h[tok], w_gu[e]), limit, alpha)
+        else:
+            act = F.gelu(F.linear(h[tok], w_gu[e]).float(), approximate="tanh" if act_kind == 2 else "none").to(h.dtype)
         y.index_add_(0, tok, wts[tok, k][:, None] * F.linear(act, w_down[e]).float())
     if shared is not None:
         y = y + shared.float()
@@ -232,13 +267,30 @@ def rotate_half_partial(x, pos, inv_freq):
     return torch.cat([a * c - b * s, b * c + a * s, x[..., 2 * half:]], -1)
 
 
-def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, ctx, k_cache, v_cache, v_first, lam):
+def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, ctx, k_cache, v_cache, v_first, lam,
+                q_head_w=None, k_head_w=None, q_head_scale=None):
     T = qkv.shape[0]
+    if k_cache is None:                        # the rows hold q only
+        q = qkv.float().reshape(T, H, D)
+        if q_head_w is not None:
+            q = _unit_rms(q, eps) * q_head_w.float()
+        if q_head_scale is not None:
+            q = q * q_head_scale.float()[None, :, None]
+        if inv_freq is not None:
+            q = rotate_half_partial(q, ctx.tok_pos, inv_freq)
+        if unit_norm:
+            q = _unit_rms(q, eps)
+        return q.to(qkv.dtype).contiguous()
     q, k, v = qkv.float().split([H * D, G * D, G * V], -1)
     if q_norm_w is not None:
         q, k = _unit_rms(q, eps) * q_norm_w.float(), _unit_rms(k, eps) * k_norm_w.float()
     q, k = q.reshape(T, H, D), k.reshape(T, G, D)
-    q, k = rotate_half_partial(q, ctx.tok_pos, inv_freq), rotate_half_partial(k, ctx.tok_pos, inv_freq)
+    if q_head_w is not None:
+        q, k = _unit_rms(q, eps) * q_head_w.float(), _unit_rms(k, eps) * k_head_w.float()
+    if q_head_scale is not None:
+        q = q * q_head_scale.float()[None, :, None]
+    if inv_freq is not None:
+        q, k = rotate_half_partial(q, ctx.tok_pos, inv_freq), rotate_half_partial(k, ctx.tok_pos, inv_freq)
     if unit_norm:
         q, k = _unit_rms(q, eps), _unit_rms(k, eps)
     if v_first is not None:
@@ -249,7 +301,23 @@ def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, c
     return q.to(qkv.dtype).contiguous()
 
 
-def paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first):
+def pool_blocks(k_cache, v_cache, kp_cache, vp_cache, pool, ctx):
+    bs, pr = k_cache.shape[1], kp_cache.shape[1]
+    kr, vr = k_cache.view(-1, *k_cache.shape[2:]), v_cache.view(-1, *v_cache.shape[2:])
+    kp, vp = kp_cache.view(-1, *kp_cache.shape[2:]), vp_cache.view(-1, *vp_cache.shape[2:])
+    for t in range(ctx.num_tokens):
+        pos, b = int(ctx.tok_pos[t]), int(ctx.tok_seq[t])
+        if (pos + 1) % pool:
+            continue
+        e = pos // pool
+        j = torch.arange(e * pool, e * pool + pool)
+        rows = ctx.block_tables[b, j // bs].long() * bs + j % bs
+        prow = int(ctx.block_tables[b, e // pr]) * pr + e % pr
+        kp[prow] = kr[rows].float().mean(0).to(kp.dtype)
+        vp[prow] = vr[rows].float().mean(0).to(vp.dtype)
+
+
+def paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first, pooled=None):
     T, H, D = q.shape
     bs, G, V = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     o = torch.empty((T, H * V), dtype=q.dtype)
@@ -270,6 +338,22 @@ def paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first):
         if window > 0:
             ok &= ((i - j[None, :]) < window) | (j[None, :] < keep_first)
         s = s.masked_fill(~ok[:, None, :], float("-inf"))
+        if pooled is not None and pooled[2] > 0:
+            kp_c, vp_c, pool = pooled
+            pr = kp_c.shape[1]
+            ne = max(0, (n - window) // pool) if n - window > 0 else 0       # entries the last token of the portion sees
+            if ne:
+                e_ = torch.arange(ne)
+                prow = ctx.block_tables[b, e_ // pr].long() * pr + e_ % pr
+                kpp = kp_c.view(-1, G, D)[prow].float().repeat_interleave(H // G, 1)
+                vpp = vp_c.view(-1, G, V)[prow].float().repeat_interleave(H // G, 1)
+                sp = torch.einsum("thd,nhd->thn", q[a:e].float(), kpp) * scale
+                seen = torch.clamp((i + 1 - window), min=0) // pool                 # [t, 1]
+                sp = sp.masked_fill(~(e_[None, :] < seen)[:, None, :], float("-inf"))
+                p = torch.softmax(torch.cat([sp, s], -1), -1)
+                o[a:e] = (torch.einsum("thn,nhv->thv", p[..., :ne], vpp) +
+                          torch.einsum("thn,nhv->thv", p[..., ne:], vv)).reshape(e - a, H * V).to(q.dtype)
+                continue
         if sink is not None:
             s = torch.cat([s, sink.float()[None, :, None].expand(e - a, H, 1)], -1)
         p = torch.softmax(s, -1)[..., :n]
@@ -315,3 +399,26 @@ def delta_gate_norm(o, g, norm_w, eps, dtype):
 
 def relu_squared(z):
     return torch.relu(z.float()).pow(2).to(z.dtype)
+
+
+def group_norm_residual(x, y, post_w, groups, eps, dtype, next_w, ids, want_h):
+    def gnorm(v, w):
+        g = v.view(v.shape[0], groups, -1)
+        return (g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)).view(v.shape) * w.float()
+    if y is not None:
+        n = gnorm((y[ids] if ids is not None else y).float(), post_w)
+        if ids is not None:
+            x = n
+        else:
+            x += n
+    if not want_h:
+        return x, None
+    h = gnorm(x, next_w).to(dtype) if next_w is not None else (x if dtype == torch.float32 else x.to(dtype))
+    return x, h
+
+
+def scale_softcap_(logits, scale, cap):
+    logits.mul_(scale)
+    if cap:
+        logits.copy_(cap * torch.tanh(logits / cap))
+    return logits

@@ -98,11 +98,13 @@ class ModelRunner:
         runner loads it, sizes the block pool and the state slots, and hands every step a StepContext."""
         cfg, hf = self.config, self.config.hf_config
         if self.on_gpu:
-            # a fresh checkout compiles the library this family runs on (and only it) here
+            # a fresh checkout compiles the libraries this family runs on (and only those) here
             import importlib
-            native = importlib.import_module("nanovllm._" + getattr(model_cls, "native_library", "seqmix"))
-            native.build_if_missing()
-            native.load()
+            names = getattr(model_cls, "native_library", "seqmix")
+            for name in ((names,) if isinstance(names, str) else names):
+                native = importlib.import_module("nanovllm._" + name)
+                native.build_if_missing()
+                native.load()
             # float32 means float32: no reduced-precision matrix mode
             torch.backends.cuda.matmul.allow_tf32 = False
         self.model = model_cls(hf)

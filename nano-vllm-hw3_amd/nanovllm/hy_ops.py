@@ -84,43 +84,79 @@ def rotary_inv_freq(dims, base, device):
 
 
 def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, ctx: StepContext, k_cache, v_cache,
-                v_first=None, lam=None):
+                v_first=None, lam=None, q_head_w=None, k_head_w=None, q_head_scale=None):
     """From the merged product qkv [T, H*D + G*D + G*V] of a step's tokens, in one launch per token:
       q_norm_w / k_norm_w given: RMS norm over the WHOLE q (k) projection with that weight;
       rotation of the first 2 * len(inv_freq) channels of every q and k head by position * inv_freq (channel i paired
       with channel i + len(inv_freq)), angles in float32;
       unit_norm: every rotated head of q and k divided by its RMS;
       v_first given: v <- (1 - lam) v + lam v_first (lam: float32 scalar on the device);
-      k and v are stored at the tokens' cache rows; returns q [T, H, D]."""
+      k and v are stored at the tokens' cache rows; returns q [T, H, D].
+    q_head_w / k_head_w [D]: before the rotation every q (k) head is divided by its own RMS and multiplied by that row,
+    shared by the heads; q_head_scale f32 [H]: query head h times its number after that.  inv_freq None: no rotation.
+    k_cache None: qkv holds q only [T, H*D] (the layer reads another layer's keys and values); nothing is stored."""
     if not qkv.is_cuda:
         return cpu_ops.qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, ctx, k_cache, v_cache,
-                                   v_first, lam)
+                                   v_first, lam, q_head_w, k_head_w, q_head_scale)
     _rows(qkv, "qkv")
     T = qkv.shape[0]
-    assert qkv.shape[1] == H * D + G * D + G * V and k_cache.dtype == v_cache.dtype == qkv.dtype
-    assert k_cache.shape[2:] == (G, D) and v_cache.shape[2:] == (G, V) and inv_freq.dtype == torch.float32
+    if k_cache is None:
+        assert qkv.shape[1] == H * D and v_cache is None
+    else:
+        assert qkv.shape[1] == H * D + G * D + G * V and k_cache.dtype == v_cache.dtype == qkv.dtype
+        assert k_cache.shape[2:] == (G, D) and v_cache.shape[2:] == (G, V)
+    assert inv_freq is None or inv_freq.dtype == torch.float32
+    assert q_head_scale is None or q_head_scale.dtype == torch.float32
     if v_first is not None:
         _rows(v_first, "v_first")
         assert v_first.shape == (T, G * V) and lam.dtype == torch.float32
     q = torch.empty((T, H, D), dtype=qkv.dtype, device=qkv.device)
     HM.check(HM.load().hm_qkv_prepare(HM.dtype_code(qkv.dtype), qkv.data_ptr(), qkv.stride(0), H, G, D, V, HM.ptr(q_norm_w),
-                                      HM.ptr(k_norm_w), float(eps), inv_freq.data_ptr(), inv_freq.numel(), int(bool(unit_norm)),
-                                      ctx.tok_pos.data_ptr(), ctx.slot_mapping.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-                                      HM.ptr(v_first), v_first.stride(0) if v_first is not None else 0, HM.ptr(lam),
-                                      q.data_ptr(), T, _dev(qkv)))
+                                      HM.ptr(k_norm_w), float(eps), HM.ptr(inv_freq), inv_freq.numel() if inv_freq is not None else 0,
+                                      int(bool(unit_norm)), ctx.tok_pos.data_ptr(), ctx.slot_mapping.data_ptr(), HM.ptr(k_cache),
+                                      HM.ptr(v_cache), HM.ptr(v_first), v_first.stride(0) if v_first is not None else 0, HM.ptr(lam),
+                                      q.data_ptr(), T, HM.ptr(q_head_w), HM.ptr(k_head_w), HM.ptr(q_head_scale), _dev(qkv)))
     return q
+
+
+def pool_rows_per_page(block_size, pool):
+    """Rows of a pooled cache page: block e of a sequence (the mean of its tokens e*pool .. e*pool + pool - 1) is row
+    e % rows of the page block_table[e // rows]; rows * pool >= block_size, so that page is the sequence's by the time
+    the block is complete."""
+    return (block_size + pool - 1) // pool
+
+
+def pool_blocks(k_cache, v_cache, kp_cache, vp_cache, pool, ctx: StepContext):
+    """For every token of the step whose position ends a block of ``pool`` tokens: the block's mean key and mean value, as
+    the caches hold them, into the pooled caches [blocks, pool_rows_per_page, G, D | V].  Call it after the step's keys
+    and values are stored."""
+    if not k_cache.is_cuda:
+        return cpu_ops.pool_blocks(k_cache, v_cache, kp_cache, vp_cache, pool, ctx)
+    bs, G, D, V = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3], v_cache.shape[3]
+    assert kp_cache.shape[1] == vp_cache.shape[1] == pool_rows_per_page(bs, pool) and kp_cache.dtype == k_cache.dtype
+    HM.check(HM.load().hm_pool_blocks(HM.dtype_code(k_cache.dtype), k_cache.data_ptr(), v_cache.data_ptr(), kp_cache.data_ptr(),
+                                      vp_cache.data_ptr(), ctx.block_tables.data_ptr(), ctx.tok_seq.data_ptr(),
+                                      ctx.tok_pos.data_ptr(), ctx.num_tokens, G, D, V, bs, ctx.block_tables.shape[1], int(pool),
+                                      kp_cache.shape[1], _dev(k_cache)))
 
 
 USE_TILES = True       # bf16 attention on the matrix cores where the shape allows (tests compare both forms)
 
 
-def paged_attention(q, k_cache, v_cache, ctx: StepContext, scale, sink=None, window=0, keep_first=0, force_rows=False):
+def paged_attention(q, k_cache, v_cache, ctx: StepContext, scale, sink=None, window=0, keep_first=0, force_rows=False,
+                    pooled=None):
     """q [T, H, D] over the paged caches k [blocks, block_size, G, D], v [blocks, block_size, G, V]; query head h reads
     key/value head h // (H/G).  The token at position i sees key j <= i, and with window > 0 only if i - j < window or
     j < keep_first.  ``sink`` f32 [H]: one more term exp(sink[h]) in the softmax denominator, without a value (zeros
-    = a sink of score 0).  Scores and weights are float32.  Returns [T, H * V]."""
+    = a sink of score 0).  Scores and weights are float32.  Returns [T, H * V].
+    ``pooled`` = (kp_cache, vp_cache, pool) with window > 0: beside its window the token also sees one key and value for
+    every block of ``pool`` tokens whose last token lies at or before i - window (the block means pool_blocks keeps), in the
+    same softmax."""
     if not q.is_cuda:
-        return cpu_ops.paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first)
+        return cpu_ops.paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first, pooled)
+    kp, vp, pool = pooled if pooled is not None else (None, None, 0)
+    pr = kp.shape[1] if kp is not None else 0
+    ptail = (HM.ptr(kp), HM.ptr(vp), int(pool), int(pr))
     HM.require_cuda(q, k_cache.dtype, "q")
     T, H, D = q.shape
     bs, G, V = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
@@ -130,21 +166,58 @@ def paged_attention(q, k_cache, v_cache, ctx: StepContext, scale, sink=None, win
     tiles_ok = (USE_TILES and not force_rows and q.dtype == torch.bfloat16 and D % 8 == 0 and V % 8 == 0 and D <= 128 and
                 V <= 128 and bs % 64 == 0)
     if tiles_ok and ctx.max_q == 1 and H // G <= 32:
-        splits = decode_splits(ctx.num_seqs * G, min(mb * bs, window + keep_first + 128) if window > 0 else mb * bs)
+        keys = min(mb * bs, window + keep_first + 128) if window > 0 else mb * bs
+        if pool:
+            keys = min(mb * bs, keys + mb * bs // pool + 64)
+        splits = decode_splits(ctx.num_seqs * G, keys)
         ws, n = HM.decode_workspace.get(q.device, lib.hm_attn_decode_workspace_bytes(T, H, V, splits))
         HM.check(lib.hm_attn_decode(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), ctx.block_tables.data_ptr(),
                                     ctx.ctx_lens.data_ptr(), HM.ptr(sink), int(window), int(keep_first), float(scale), o.data_ptr(),
-                                    T, H, G, D, V, bs, mb, splits, ws, n, _dev(q)))
+                                    T, H, G, D, V, bs, mb, splits, ws, n, *ptail, _dev(q)))
         return o
     if tiles_ok:
         HM.check(lib.hm_attn_tiles(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), ctx.block_tables.data_ptr(),
                                    ctx.qstart.data_ptr(), ctx.seq_pos0.data_ptr(), HM.ptr(sink), int(window), int(keep_first),
-                                   float(scale), o.data_ptr(), ctx.num_seqs, ctx.max_q, H, G, D, V, bs, mb, _dev(q)))
+                                   float(scale), o.data_ptr(), ctx.num_seqs, ctx.max_q, H, G, D, V, bs, mb, *ptail, _dev(q)))
         return o
     HM.check(lib.hm_attn_rows(HM.dtype_code(q.dtype), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                               ctx.block_tables.data_ptr(), ctx.tok_seq.data_ptr(), ctx.tok_pos.data_ptr(), HM.ptr(sink),
-                              int(window), int(keep_first), float(scale), o.data_ptr(), T, H, G, D, V, bs, mb, _dev(q)))
+                              int(window), int(keep_first), float(scale), o.data_ptr(), T, H, G, D, V, bs, mb, *ptail, _dev(q)))
     return o
+
+
+def group_norm_residual(x, y, post_w, groups, eps, dtype, next_w=None, ids=None, want_h=True):
+    """The boundary between two sublayers of a float32 residual x [T, W] that is normalised on the sublayers' OUTPUT, the
+    RMS norm taken over ``groups`` equal consecutive parts of the vector; per token in one launch:
+      y given:        x <- x + group_norm(y) * post_w   (ids given: x <- group_norm(y[ids]) * post_w, y an embedding table;
+                      x may then be None and is made here)
+      want_h:         returns group_norm(x) * next_w if next_w is given, else x itself, in ``dtype`` (what the next
+                      sublayer, or the vocabulary product, reads); for float32 without next_w that is x, no copy.
+    Returns (x, h)."""
+    on_cpu = not (y if y is not None else x).is_cuda
+    if on_cpu:
+        return cpu_ops.group_norm_residual(x, y, post_w, groups, eps, dtype, next_w, ids, want_h)
+    T = ids.numel() if ids is not None else (y if y is not None else x).shape[0]
+    W = (y if y is not None else x).shape[1]
+    if x is None:
+        x = torch.empty((T, W), dtype=torch.float32, device=y.device)
+    if y is not None:
+        HM.require_cuda(y, dtype, "y")
+    h = None
+    if want_h and (next_w is not None or dtype != torch.float32):
+        h = torch.empty((T, W), dtype=dtype, device=x.device)
+    HM.check(HM.load().hm_group_norm_residual(HM.dtype_code(dtype), x.data_ptr(), HM.ptr(y), HM.ptr(ids), HM.ptr(post_w),
+                                              HM.ptr(next_w), int(groups), float(eps), HM.ptr(h), T, W, _dev(x)))
+    return x, (h if h is not None or not want_h else x)
+
+
+def scale_softcap_(logits, scale, cap):
+    """logits f32, in place: cap * tanh(logits * scale / cap) (cap <= 0 or None: logits * scale)."""
+    if not logits.is_cuda:
+        return cpu_ops.scale_softcap_(logits, scale, cap)
+    assert logits.dtype == torch.float32 and logits.is_contiguous()
+    HM.check(HM.load().hm_scale_softcap(logits.data_ptr(), logits.numel(), float(scale), float(cap or 0.0), _dev(logits)))
+    return logits
 
 
 def decode_splits(num_groups, max_keys):

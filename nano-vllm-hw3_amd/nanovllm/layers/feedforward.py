@@ -37,24 +37,38 @@ class ClampedGLU(nn.Module):
 class RoutedExperts(nn.Module):
     """Softmax router in float32; experts in ``groups`` equal groups of neighbours, only the ``keep`` groups with the
     largest member score are eligible; the ``top`` best eligible experts run, weighted by their renormalised scores.
-    A shared expert (its own size and limit) runs for every token and is added."""
+    A shared expert (its own size and limit) runs for every token and is added.
 
-    def __init__(self, width: int, experts: int, top: int, ff: int, limit: float, groups: int = 1, keep: int = 1,
-                 shared: ClampedGLU = None, alpha: float = 1.702):
+    Variations: ``score`` = "sigmoid" (independent scores instead of a softmax); ``correction``: a learned per-expert
+    number added to the scores for the CHOICE of groups and experts only (the weights stay the scores); ``group_top``: a
+    group scores the sum of that many of its largest choice scores instead of the largest; ``renorm`` = False: the chosen
+    scores weigh as they are; ``act`` = "gelu" / "gelu_tanh": an expert is down(gelu(up h)), no gate, no clamp."""
+
+    ACTS = {"clamped_glu": seq_ops.ACT_CLAMPED_GLU, "gelu": seq_ops.ACT_GELU, "gelu_tanh": seq_ops.ACT_GELU_TANH}
+
+    def __init__(self, width: int, experts: int, top: int, ff: int, limit: float = 0.0, groups: int = 1, keep: int = 1,
+                 shared: ClampedGLU = None, alpha: float = 1.702, score: str = "softmax", correction: bool = False,
+                 group_top: int = 1, renorm: bool = True, act: str = "clamped_glu"):
         super().__init__()
         self.experts, self.top, self.groups, self.keep, self.limit, self.alpha = experts, top, groups, keep, float(limit), alpha
+        self.score = {"softmax": seq_ops.ROUTE_SOFTMAX, "sigmoid": seq_ops.ROUTE_SIGMOID}[score]
+        self.group_top, self.renorm, self.act_kind = group_top, renorm, self.ACTS[act]
+        self.parts = 2 if act == "clamped_glu" else 1           # gate and up rows, or up rows alone
+        self.correction = nn.Parameter(torch.zeros(experts, dtype=torch.float32), requires_grad=False) if correction else None
         self.router = nn.Parameter(torch.empty(experts, width, dtype=torch.float32), requires_grad=False)
-        self.w_gu = nn.Parameter(torch.empty(experts, 2 * ff, width), requires_grad=False)
+        self.w_gu = nn.Parameter(torch.empty(experts, self.parts * ff, width), requires_grad=False)
         self.w_down = nn.Parameter(torch.empty(experts, width, ff), requires_grad=False)
         self.shared = shared
         self._tiled = None         # the expert weights in the layout the matrix-core kernels stream (made at the first step)
 
     def forward(self, h):
         if self._tiled is None and h.is_cuda and h.dtype == torch.bfloat16:
-            self._tiled = (seq_ops.tile_expert_weights(self.w_gu, 2), seq_ops.tile_expert_weights(self.w_down))
-        idx, wts = seq_ops.moe_route(h, self.router, self.top, self.groups, self.keep)
+            self._tiled = (seq_ops.tile_expert_weights(self.w_gu, self.parts), seq_ops.tile_expert_weights(self.w_down))
+        idx, wts = seq_ops.moe_route(h, self.router, self.top, self.groups, self.keep, self.score, self.correction,
+                                     self.group_top, self.renorm)
         shared = self.shared(h) if self.shared is not None else None
-        return seq_ops.moe_experts(h, idx, wts, self.w_gu, self.w_down, self.limit, self.alpha, shared, tiled=self._tiled)
+        return seq_ops.moe_experts(h, idx, wts, self.w_gu, self.w_down, self.limit, self.alpha, shared, tiled=self._tiled,
+                                   act_kind=self.act_kind)
 
 
 class ReluSquaredMLP(nn.Module):

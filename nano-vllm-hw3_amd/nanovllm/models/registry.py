@@ -11,6 +11,7 @@ _MODELS = {
     "Qwen2ForCausalLM": ("nanovllm.models.qwen3", "Qwen3ForCausalLM"),      # the same decoder with qkv biases
     "Pasizen": ("nanovllm.models.pasizen", "PasizenForCausalLM"),
     "Lipelix": ("nanovllm.models.lipelix", "LipelixForCausalLM"),
+    "Galupel": ("nanovllm.models.galupel", "GalupelForCausalLM"),
 }
 DEFAULT = "Qwen3ForCausalLM"
 

@@ -100,33 +100,51 @@ def latent_norm_store(x, w, eps, cache, slot_mapping):
                                             cache.data_ptr(), slot_mapping.data_ptr(), T, R, _dev(x)))
 
 
+def latent_rope_store(x, w, eps, q, qa, inv_freq, rot_dims, H, D, R, Rd, cache, ctx: StepContext):
+    """A latent with a rotated key part.  x [T, R + Rd] (rows may be a column slice): rms_norm(x[:, :R]) * w and x[:, R:]
+    with its first rot_dims channels turned by position * inv_freq (channel 2i pairs with 2i + 1) are stored as the
+    tokens' rows of ``cache`` [blocks, block_size, R + Rd].  q [T, H * (D + Rd)] (rows may be a slice): every head's last
+    Rd channels, turned the same way, go to qa[:, :, R:] (qa [T, H, R + Rd]; its first R columns are the caller's)."""
+    if not x.is_cuda:
+        return cpu_ops.latent_rope_store(x, w, eps, q, qa, inv_freq, rot_dims, H, D, R, Rd, cache, ctx)
+    T = x.shape[0]
+    assert x.stride(1) == 1 and q.stride(1) == 1 and qa.is_contiguous() and x.dtype == cache.dtype == w.dtype == q.dtype == qa.dtype
+    assert x.shape[1] == R + Rd and q.shape[1] == H * (D + Rd) and qa.shape == (T, H, R + Rd) and cache.shape[2] == R + Rd
+    SM.check(SM.load().sm_latent_rope_store(SM.dtype_code(x.dtype), x.data_ptr(), x.stride(0), w.data_ptr(), eps, q.data_ptr(),
+                                            q.stride(0), qa.data_ptr(), SM.ptr(inv_freq), rot_dims, ctx.tok_pos.data_ptr(),
+                                            cache.data_ptr(), ctx.slot_mapping.data_ptr(), T, H, D, R, Rd, _dev(x)))
+
+
 USE_TILES = True       # bf16 latent attention on the matrix cores where the shape allows (tests compare both forms)
 
 
-def latent_attention(q, cache, ctx: StepContext, scale, force_rows=False):
-    """Absorbed queries q [T, H, R] over the paged latent cache [blocks, block_size, R] (keys = values = cache rows),
-    causal inside each sequence -> [T, H, R]."""
+def latent_attention(q, cache, ctx: StepContext, scale, force_rows=False, value_cols=0, window=0):
+    """Absorbed queries q [T, H, R] over the paged latent cache [blocks, block_size, R], causal inside each sequence.
+    A cache row is the key; its first ``value_cols`` columns are the value (0 = all of it) -> [T, H, value_cols or R].
+    ``window`` > 0: the token at position i sees only the keys j with i - j < window."""
     T, H, R = q.shape
+    RV = value_cols or R
     if not q.is_cuda:
-        return cpu_ops.latent_attention(q, cache, ctx, scale)
+        return cpu_ops.latent_attention(q, cache, ctx, scale, RV, window)
     SM.require_cuda(q, cache.dtype, "q")
-    o = torch.empty_like(q)
+    o = torch.empty((T, H, RV), dtype=q.dtype, device=q.device)
     lib = SM.load()
     bs, mb = cache.shape[1], ctx.block_tables.shape[1]
-    tiles_ok = (USE_TILES and not force_rows and q.dtype == torch.bfloat16 and R % 8 == 0 and R <= 256 and bs % 64 == 0)
+    tiles_ok = (USE_TILES and not force_rows and q.dtype == torch.bfloat16 and R % 8 == 0 and RV % 4 == 0 and R <= 256 and
+                bs % 64 == 0)
     if tiles_ok and ctx.max_q == 1 and H <= 128:
-        splits = decode_splits(ctx.num_seqs, mb * bs)
+        splits = decode_splits(ctx.num_seqs, min(mb * bs, window + 64) if window > 0 else mb * bs)
         ws, n = SM.decode_workspace.get(q.device, lib.sm_latent_decode_workspace_bytes(T, H, R, splits))
         SM.check(lib.sm_latent_attn_decode(q.data_ptr(), cache.data_ptr(), ctx.block_tables.data_ptr(), ctx.ctx_lens.data_ptr(),
-                                           o.data_ptr(), scale, T, H, R, bs, mb, splits, ws, n, _dev(q)))
+                                           o.data_ptr(), scale, T, H, R, bs, mb, splits, ws, n, RV, int(window), _dev(q)))
     elif tiles_ok:
         SM.check(lib.sm_latent_attn_tiles(q.data_ptr(), cache.data_ptr(), ctx.block_tables.data_ptr(), ctx.qstart.data_ptr(),
                                           ctx.seq_pos0.data_ptr(), o.data_ptr(), scale, ctx.num_seqs, ctx.max_q, H, R, bs, mb,
-                                          _dev(q)))
+                                          RV, int(window), _dev(q)))
     else:
         SM.check(lib.sm_latent_attn_rows(SM.dtype_code(q.dtype), q.data_ptr(), cache.data_ptr(), ctx.block_tables.data_ptr(),
                                          ctx.tok_seq.data_ptr(), ctx.tok_pos.data_ptr(), o.data_ptr(), scale, T, H, R, bs, mb,
-                                         _dev(q)))
+                                         RV, int(window), _dev(q)))
     return o
 
 
@@ -159,10 +177,19 @@ def clamped_glu(gu, limit, alpha=1.702):
     return out
 
 
-def moe_route(h, router_w, top, groups=1, keep=1):
-    """Softmax router with group-limited top-k: (idx int32 [T, top], weights f32 [T, top]); router_w f32 [E, W]."""
+ROUTE_SOFTMAX, ROUTE_SIGMOID = 0, 1
+ACT_CLAMPED_GLU, ACT_GELU, ACT_GELU_TANH = 0, 1, 2
+
+
+def moe_route(h, router_w, top, groups=1, keep=1, score=ROUTE_SOFTMAX, correction=None, group_top=1, renorm=True):
+    """Router with group-limited top-k: (idx int32 [T, top], weights f32 [T, top]); router_w f32 [E, W].  Scores are the
+    softmax or the sigmoid of the float32 logits; ``correction`` f32 [E] is added for the CHOICE only (groups and
+    experts), the weights stay the scores; a group scores the sum of its ``group_top`` largest choice scores (1 = its
+    maximum); ``renorm``: the chosen weights are divided by their sum."""
     if not h.is_cuda:
-        return cpu_ops.moe_route(h, router_w, top, groups, keep)
+        return cpu_ops.moe_route(h, router_w, top, groups, keep, score, correction, group_top, renorm)
+    if correction is not None:
+        SM.require_cuda(correction, torch.float32, "correction")
     SM.require_cuda(h, None, "h")
     SM.require_cuda(router_w, torch.float32, "router_w")
     T, W = h.shape
@@ -170,7 +197,8 @@ def moe_route(h, router_w, top, groups=1, keep=1):
     idx = torch.empty((T, top), dtype=torch.int32, device=h.device)
     wts = torch.empty((T, top), dtype=torch.float32, device=h.device)
     SM.check(SM.load().sm_moe_route(SM.dtype_code(h.dtype), h.data_ptr(), router_w.data_ptr(), idx.data_ptr(), wts.data_ptr(),
-                                    T, W, E, top, groups, keep, _dev(h)))
+                                    T, W, E, top, groups, keep, int(score), SM.ptr(correction), int(group_top), int(bool(renorm)),
+                                    _dev(h)))
     return idx, wts
 
 
@@ -190,14 +218,17 @@ def tile_expert_weights(w, parts=1):
     return x.contiguous()
 
 
-def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form=None, tiled=None):
+def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form=None, tiled=None, act_kind=ACT_CLAMPED_GLU):
     """y[t] = sum_k wts[t, k] * expert_{idx[t, k]}(h[t]) (+ shared[t]); w_gu [E, 2F, W] (gate rows then up rows),
     w_down [E, W, F]; an expert is a clamped GLU between its two products.  ``form``: "pairs" | "grouped" | "tiles128"
     forces one; by default float32 runs pair by pair and bf16 grouped by expert on the matrix cores, in tiles of 32 rows
     for small groups (decode) and of 128 rows for large ones (prefill).  ``tiled`` = (tile_expert_weights(w_gu, 2),
-    tile_expert_weights(w_down)), what the grouped forms read (made here when the caller does not keep them)."""
+    tile_expert_weights(w_down)), what the grouped forms read (made here when the caller does not keep them).
+    ``act_kind`` = ACT_GELU / ACT_GELU_TANH: an expert is down(gelu(up h)) instead, w_gu is [E, F, W] (tiled in one part)."""
     if not h.is_cuda:
-        return cpu_ops.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared)
+        return cpu_ops.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared, act_kind)
+    parts = 2 if act_kind == ACT_CLAMPED_GLU else 1
+    assert w_gu.shape[1] == parts * w_down.shape[2]
     SM.require_cuda(h, w_gu.dtype, "h")
     T, W = h.shape
     top, F = idx.shape[1], w_down.shape[2]
@@ -217,16 +248,16 @@ def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form
         prod = torch.empty((rows * n, W), dtype=h.dtype, device=h.device)
         act = torch.empty((rows * n, F), dtype=h.dtype, device=h.device)
         fn = lib.sm_moe_grouped if form == "grouped" else lib.sm_moe_tiles128
-        t_gu, t_down = tiled if tiled is not None else (tile_expert_weights(w_gu, 2), tile_expert_weights(w_down))
+        t_gu, t_down = tiled if tiled is not None else (tile_expert_weights(w_gu, parts), tile_expert_weights(w_down))
         SM.check(fn(h.data_ptr(), idx.data_ptr(), wts.data_ptr(), t_gu.data_ptr(), t_down.data_ptr(), SM.ptr(shared), limit, alpha,
-                    y.data_ptr(), T, top, E, W, F, row_pair.data_ptr(), tile_expert.data_ptr(), pair_row.data_ptr(),
+                    int(act_kind), y.data_ptr(), T, top, E, W, F, row_pair.data_ptr(), tile_expert.data_ptr(), pair_row.data_ptr(),
                     act.data_ptr(), prod.data_ptr(), _dev(h)))
         return y
     assert form == "pairs", form
     act = torch.empty((T * top, F), dtype=h.dtype, device=h.device)
     y = torch.empty_like(h)
-    SM.check(lib.sm_moe_pairs_gate_up(code, h.data_ptr(), idx.data_ptr(), w_gu.data_ptr(), limit, alpha, act.data_ptr(), T, top,
-                                      W, F, _dev(h)))
+    SM.check(lib.sm_moe_pairs_gate_up(code, h.data_ptr(), idx.data_ptr(), w_gu.data_ptr(), limit, alpha, int(act_kind),
+                                      act.data_ptr(), T, top, W, F, _dev(h)))
     SM.check(lib.sm_moe_pairs_down(code, act.data_ptr(), idx.data_ptr(), wts.data_ptr(), w_down.data_ptr(), SM.ptr(shared),
                                    y.data_ptr(), T, top, W, F, _dev(h)))
     return y
