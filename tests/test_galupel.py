@@ -1,0 +1,367 @@
+"""The Galupel model family in the engine against the plain restatement in tests/oracle_galupel.py.
+
+Every test makes its own small configuration and random checkpoint.  ``device`` = "cpu" drives the engine's plumbing
+operators (scheduler, block and slot pools, portion batching are the same code as on the GPU); "cuda" (marked gpu) drives
+the HIP kernels of libhymix and libseqmix, in float32 against tight bounds and in bfloat16 against the rounding of that
+format."""
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "nano-vllm-hw3_amd"))
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+import oracle_galupel as O  # noqa: E402
+from test_pasizen import DEVICES, cut, dtypes_for, replay, tokens, write_model  # noqa: E402  (engine test helpers)
+
+
+def attn(heads=4, kv_heads=2, dim=16, vdim=8, scale=0.3, window=9, pool=4, kv_from=None):
+    m = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=scale, mask=dict(size=window, pool=pool))
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return "attention", m
+
+
+def latent(heads=3, dim=8, rot_dim=8, vdim=16, kv_rank=24, scale=0.3, window=21, base=50.0, dims=None):
+    return "latent_attention", dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim, kv_rank=kv_rank, scale=scale,
+                                    rot=dict(dims=rot_dim if dims is None else dims, base=base), mask=dict(size=window))
+
+
+def moe(experts=8, top=3, ff=24, groups=(4, 2)):
+    return dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, top=top, groups=dict(count=groups[0], keep=groups[1])))
+
+
+def config(layers, width=48, vocab=61, eps=1e-5, groups=3, logit_scale=1.5, softcap=20.0):
+    return dict(architecture="Galupel", vocab=vocab, width=width, norm=dict(eps=eps, groups=groups), logit_scale=logit_scale,
+                logit_softcap=softcap, layers=[dict(type=kind, mixer=m, mlp=mlp) for (kind, m), mlp in layers])
+
+
+DEFAULT = [(latent(), moe()), (attn(), moe(experts=6, top=2, ff=16, groups=(3, 2))), (attn(heads=2, kv_heads=1, dim=24, vdim=24, window=70, pool=3), None),
+           (latent(heads=2, dim=16, rot_dim=4, vdim=8, kv_rank=40, window=64), None), (attn(window=5, pool=4, kv_from=1), moe(experts=4, top=1, groups=(1, 1)))]
+
+
+def weights(cfg, seed=0, temp=0.3):
+    """A random checkpoint under the design's tensor names, bf16-representable values."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+
+    def rnd(*shape, s=1.0):
+        return (torch.randn(*shape, generator=g) * s).to(torch.bfloat16)
+    t = {"embed": rnd(cfg["vocab"], W, s=0.5), "embed.norm": 1 + rnd(W, s=0.1), "final.norm": 1 + rnd(W, s=0.1)}
+    for i, L in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        H, D, V = m["heads"], m["dim"], m["vdim"]
+        t[p + "norm1"] = 0.5 + rnd(W, s=0.1)
+        if L["type"] == "attention":
+            G = m["kv_heads"]
+            t.update({p + "mix.q": rnd(H * D, W, s=W ** -0.5), p + "mix.q.norm": 1.5 + rnd(D, s=0.3),
+                      p + "mix.temp": 1 + rnd(H, s=temp), p + "mix.o": rnd(W, H * V, s=(H * V) ** -0.5)})
+            if m.get("kv_from") is None:
+                t.update({p + "mix.k": rnd(G * D, W, s=W ** -0.5), p + "mix.v": rnd(G * V, W, s=W ** -0.5),
+                          p + "mix.k.norm": 1.5 + rnd(D, s=0.3)})
+        else:
+            R, Rd = m["kv_rank"], m["rot_dim"]
+            t.update({p + "mix.q": rnd(H * (D + Rd), W, s=2 * W ** -0.5), p + "mix.dkv": rnd(R + Rd, W, s=2 * W ** -0.5),
+                      p + "mix.dkv.norm": 1 + rnd(R, s=0.2), p + "mix.uk": rnd(H * D, R, s=R ** -0.5),
+                      p + "mix.uv": rnd(H * V, R, s=R ** -0.5), p + "mix.o": rnd(W, H * V, s=(H * V) ** -0.5)})
+        if L["mlp"] is not None:
+            E, ff = L["mlp"]["router"]["experts"], L["mlp"]["expert"]["ff"]
+            t.update({p + "norm2": 0.5 + rnd(W, s=0.1), p + "mlp.router": rnd(E, W, s=3 * W ** -0.5),
+                      p + "mlp.correction": rnd(E, s=0.4)})
+            for e in range(E):
+                t.update({f"{p}mlp.e{e}.up": rnd(ff, W, s=2 * W ** -0.5), f"{p}mlp.e{e}.down": rnd(W, ff, s=ff ** -0.5)})
+    return {k: v.to(torch.bfloat16).contiguous() for k, v in t.items()}
+
+
+def close(got, ref, dtype, frac=0.0):
+    """Logit rows against the oracle's (difference with its mean removed, relative to the spread of the logits): float32
+    to accumulation order, bfloat16 to that format's rounding through the layers.  ``frac``: the share of rows that may
+    lie outside (bfloat16 only: a router's near-tie may turn under rounding and swap an expert for that token)."""
+    got, ref = np.asarray(got, dtype=np.float64), np.asarray(ref, dtype=np.float64)
+    assert got.shape == ref.shape and np.isfinite(got).all()
+    d = got - ref
+    d = d - d.mean(-1, keepdims=True)
+    err = np.sqrt((d ** 2).mean(-1)) / ref.std()
+    bound = 2e-4 if dtype == torch.float32 else 6e-2
+    bad = (err >= bound).mean()
+    allowed = frac if dtype == torch.bfloat16 else 0.0
+    assert bad <= allowed, f"{bad:.3f} of the rows beyond {bound}; relative error {err.max():.3g} at row {int(err.argmax())}"
+
+
+BF16_TIES = 0.08       # share of rows a turned near-tie of these small random routers may move in bfloat16
+
+
+@pytest.fixture(scope="module")
+def model(tmp_path_factory):
+    cfg = config(DEFAULT)
+    w = weights(cfg, seed=1)
+    return write_model(tmp_path_factory.mktemp("galupel_default"), cfg, w), cfg, w
+
+
+def forward(cfg, w, toks, **kw):
+    return O.forward(cfg, w, toks, **kw).numpy()
+
+
+# ------------------------------------------------------------------------------------------ whole model, schedules
+@pytest.mark.parametrize("device", DEVICES)
+def test_whole_prompt_and_layer_trace(model, tmp_path, device):
+    """One step per prompt: every position's logits; and the residual after every layer, through the runner itself."""
+    path, cfg, w = model
+    toks = tokens(90, cfg["vocab"], 3)
+    layers = []
+    ref = forward(cfg, w, toks, layers_out=layers)
+    for dtype in dtypes_for(device):
+        got = replay(path, [([("a", toks, list(range(90)))], ["a"])], tmp_path, device, dtype)
+        close(got[0], ref, dtype, BF16_TIES)
+    from nanovllm.engine.llm_engine import LLMEngine
+    from nanovllm.engine.sequence import ACTIVE, Sequence
+    eng = LLMEngine(path, device=device, dtype=torch.float32, max_num_seqs=2, num_kvcache_blocks=4, max_num_batched_tokens=4096)
+    seq = Sequence(toks)
+    seq.state = ACTIVE
+    assert eng.scheduler.reserve_portion(seq, 90)
+    trace = []
+    eng.model_runner.run_portions([(seq, 90)], trace=trace)
+    assert len(trace) == len(layers) == 5
+    for got_l, ref_l in zip(trace, layers):
+        assert torch.allclose(got_l.cpu().double(), ref_l, atol=2e-4, rtol=2e-4)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_prefill_equals_token_by_token(model, tmp_path, device):
+    """A prompt fed one token per step (caches and pooled blocks built from the very first token) gives the logits of the
+    whole prompt in one step; 150 tokens cross two cache-block borders, every window and many pooled blocks."""
+    path, cfg, w = model
+    toks = tokens(150, cfg["vocab"], 4)
+    ref = forward(cfg, w, toks)
+    steps = [([("a", [t], [0])], ["a"] if i == 149 else []) for i, t in enumerate(toks)]
+    for dtype in dtypes_for(device):
+        got = replay(path, steps, tmp_path, device, dtype, max_tokens=192)
+        close(np.concatenate([got[i] for i in range(150)]), ref, dtype, BF16_TIES)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("sizes", [[2], [3, 2, 7, 2, 64, 1, 5], [63, 2, 1, 64], [65, 1, 1, 1, 2], [9, 1, 8, 10]])
+def test_portions(model, tmp_path, device, sizes):
+    """Prompts cut into portions of several sizes (down to two tokens, across cache-block borders, window edges and the
+    ends of pooled blocks, single tokens between): a pooled block may be completed by a later step than it was begun in."""
+    path, cfg, w = model
+    toks = tokens(133, cfg["vocab"], 5)
+    ref = forward(cfg, w, toks)
+    parts = cut(133, sizes)
+    steps = [([("r", toks[a:b], list(range(b - a)))], ["r"] if b == 133 else []) for a, b in parts]
+    for dtype in dtypes_for(device):
+        got = replay(path, steps, tmp_path, device, dtype, max_tokens=192)
+        close(np.concatenate([got[i] for i in range(len(parts))]), ref, dtype, BF16_TIES)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_mixed_batches_and_reused_pages(model, tmp_path, device):
+    """Unequal requests share steps (prompt portions beside single tokens), more requests than slots and more tokens than
+    cache blocks over the run: blocks (with the pooled rows that belong to them) and slots are freed and taken again.
+    Each request equals itself alone."""
+    path, cfg, w = model
+    V = cfg["vocab"]
+    reqs = {f"q{i}": tokens(n, V, 10 + i) for i, n in enumerate([97, 5, 130, 66, 1, 71, 64])}
+    ref = {k: forward(cfg, w, v) for k, v in reqs.items()}
+    plan = {"q0": cut(97, [40, 1, 1, 30, 1]), "q1": cut(5, [2, 1]), "q2": cut(130, [64, 3, 1]), "q3": cut(66, [66]),
+            "q4": cut(1, [1]), "q5": cut(71, [7, 1]), "q6": cut(64, [62, 2])}
+    live, waiting, steps, rows = [], list(reqs), [], []
+    cursor = {k: 0 for k in reqs}
+    while live or waiting:
+        while waiting and len(live) < 3:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for k in list(live):
+            a, b = plan[k][cursor[k]]
+            cursor[k] += 1
+            entries.append((k, reqs[k][a:b], list(range(b - a))))
+            rows.append((len(steps), k, a, b))
+            if b == len(reqs[k]):
+                end.append(k)
+                live.remove(k)
+        steps.append((entries, end))
+    for dtype in dtypes_for(device):
+        got = replay(path, steps, tmp_path, device, dtype, max_tokens=7 * 64, max_live=3)
+        at, all_got, all_ref = {}, [], []
+        for s, k, a, b in rows:
+            o = at.get(s, 0)
+            all_got.append(got[s][o:o + b - a])
+            all_ref.append(ref[k][a:b])
+            at[s] = o + b - a
+        close(np.concatenate(all_got), np.concatenate(all_ref), dtype, BF16_TIES)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_long_decoding(model, tmp_path, device):
+    """A short prompt and 200 single-token steps: three block borders, every window and dozens of pooled blocks pass over
+    decoded tokens."""
+    path, cfg, w = model
+    toks = tokens(215, cfg["vocab"], 6)
+    ref = forward(cfg, w, toks)
+    steps = [([("a", toks[:15], [14])], [])] + [([("a", [t], [0])], []) for t in toks[15:]]
+    for dtype in dtypes_for(device):
+        got = replay(path, steps, tmp_path, device, dtype, max_tokens=256)
+        close(np.concatenate([got[i] for i in range(len(steps))]), ref[14:], dtype, BF16_TIES)
+
+
+VARIANTS = {
+    # sizes that the default makes equal are unequal here and the other way round; values of 1
+    "attention_only_one_head_window_1": config([(attn(heads=1, kv_heads=1, dim=8, vdim=8, window=1, pool=1), None)], groups=1, softcap=0.0),
+    "latent_only_top_1_ungrouped": config([(latent(heads=1, dim=4, rot_dim=2, vdim=4, kv_rank=8, window=1), moe(experts=5, top=1, groups=(1, 1)))],
+                                          width=16, groups=16, logit_scale=1.0),
+    "pool_wider_than_a_page": config([(attn(window=3, pool=70), moe(experts=4, top=4, groups=(2, 2))), (attn(window=64, pool=64, kv_from=0), None),
+                                      (attn(window=65, pool=2, kv_from=0), None)], groups=2),
+    "window_of_a_page_and_more": config([(latent(window=64, dims=4), None), (latent(window=65, rot_dim=12, kv_rank=36, dim=4), moe(groups=(2, 1), top=2)),
+                                         (latent(window=200), None)], width=24, groups=4),
+    "big_heads": config([(attn(heads=2, kv_heads=2, dim=72, vdim=40, window=33, pool=5), None), (latent(heads=2, dim=40, rot_dim=24, vdim=72, kv_rank=136, window=50), None)]),
+}
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("name", sorted(VARIANTS))
+def test_other_shapes(tmp_path, device, name):
+    """Other sizes, orders and constants: each mixer alone, one head, windows of one token / of a cache block / one more /
+    longer than the prompt, pooled blocks of one token and of more than a cache block, readers whose block size differs
+    from their source's, rotation of part of the rotated part, a norm over one group and over groups of one channel, top 1
+    and all experts, one group, one kept group, no soft cap, sizes off the matrix-core tiles.  Portions and a batch."""
+    cfg = VARIANTS[name]
+    w = weights(cfg, seed=7)
+    path = write_model(tmp_path / "m", cfg, w)
+    a, b = tokens(150, cfg["vocab"], 8), tokens(9, cfg["vocab"], 9)
+    ra, rb = forward(cfg, w, a), forward(cfg, w, b)
+    steps = [([("a", a[:31], list(range(31)))], []),
+             ([("a", a[31:131], list(range(100))), ("b", b[:2], [0, 1])], []),
+             ([("b", b[2:], list(range(7))), ("a", a[131:132], [0])], ["b"])] + \
+            [([("a", [t], [0])], []) for t in a[132:]]
+    for dtype in dtypes_for(device):
+        got = replay(path, steps, tmp_path, device, dtype, max_tokens=256)
+        allg = np.concatenate([got[i] for i in range(len(steps))])
+        allr = np.concatenate([ra[:31], ra[31:131], rb[:2], rb[2:], ra[131:132], ra[132:]])
+        close(allg, allr, dtype, BF16_TIES)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_far_blocks_and_window_edges_show(tmp_path, device):
+    """Weights made so that faults show: a token's key is its first head's query and the scores are steep, so equal tokens
+    attract.  A token repeated far back reaches the query only through its pooled block (whose mean then leans to it); a
+    token just inside the window attracts by itself, one just outside only if its block is already seen.  A lost block, a
+    window one token off or a block seen one token early moves these rows by much more than the bound."""
+    cfg = config([(attn(heads=2, kv_heads=1, dim=16, vdim=16, scale=6.0, window=10, pool=3), None)], width=32, groups=1)
+    w = weights(cfg, seed=3, temp=0.0)
+    w["l0.mix.k"] = w["l0.mix.q"][:16].clone()
+    w["l0.mix.k.norm"] = w["l0.mix.q.norm"].clone()
+    path = write_model(tmp_path / "m", cfg, w)
+    toks = tokens(300, cfg["vocab"], 12)
+    # the query at `at` meets its own token at: a far pooled block, a block border of the cache, the last position inside
+    # the window (at - 9), the first outside (at - 10), and the last token of the newest seen / the oldest unseen block
+    for far, at in ((2, 290), (63, 291), (64, 292), (129, 293), (294 - 9, 294), (295 - 10, 295), (280, 296), (284, 297)):
+        toks[far] = toks[at]
+    ref = forward(cfg, w, toks)
+    wrong = O.forward(dict(cfg, layers=[dict(cfg["layers"][0], mixer=dict(cfg["layers"][0]["mixer"], mask=dict(size=10, pool=0)))]), w, toks).numpy()
+    assert np.abs(ref[290:298] - wrong[290:298]).max() > 0.05 * ref.std()      # the pooled blocks matter in this model
+    steps = [([("a", toks[:280], [279])], [])] + [([("a", [t], [0])], []) for t in toks[280:]]
+    for dtype in dtypes_for(device):
+        got = replay(path, steps, tmp_path, device, dtype, max_tokens=320)
+        close(np.concatenate([got[i] for i in range(len(steps))]), ref[279:], dtype)
+        whole = replay(path, [([("a", toks, list(range(270, 300)))], ["a"])], tmp_path, device, dtype, max_tokens=320)
+        close(whole[0], ref[270:], dtype)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_greedy_generation_through_the_scheduler(model, device):
+    """LLM.generate (the scheduler's own portions: a 16-token step budget cuts prompts, decoded tokens share steps with
+    prompt pieces, five requests over three slots) continues every prompt as the oracle's greedy loop does."""
+    from nanovllm import LLM, SamplingParams
+    path, cfg, w = model
+    prompts = [tokens(n, cfg["vocab"], 20 + n) for n in (37, 3, 18, 1, 70)]
+
+    def greedy(p, n):
+        p = list(p)
+        for _ in range(n):
+            p.append(int(forward(cfg, w, p)[-1].argmax()))
+        return p[-n:]
+    llm = LLM(path, device=device, dtype=torch.float32, max_num_seqs=3, max_num_batched_tokens=16, num_kvcache_blocks=5)
+    out = llm.generate(prompts, SamplingParams(max_tokens=6, ignore_eos=True))
+    assert [o["token_ids"] for o in out] == [greedy(p, 6) for p in prompts]
+    assert len(llm.scheduler.block_manager.free) == 5 and len(llm.scheduler.slots.free) == 3
+
+
+def test_scheduler_preempts_when_blocks_run_out(model):
+    """Two requests that cannot both grow in a three-block pool: the later one is put back, runs again afterwards from
+    its first token (its pages hold another request's rows by then), and both produce what they produce alone."""
+    from nanovllm import LLM, SamplingParams
+    path, cfg, w = model
+    prompts = [tokens(60, cfg["vocab"], 31), tokens(62, cfg["vocab"], 32)]
+    sp = SamplingParams(max_tokens=10, ignore_eos=True)
+    alone = [LLM(path, device="cpu", dtype=torch.float32, max_num_seqs=2, num_kvcache_blocks=4).generate([p], sp)[0]["token_ids"]
+             for p in prompts]
+    llm = LLM(path, device="cpu", dtype=torch.float32, max_num_seqs=2, num_kvcache_blocks=3)
+    out = llm.generate(prompts, sp)
+    assert [o["token_ids"] for o in out] == alone
+
+
+def test_registry_config_and_dummy_weights(tmp_path):
+    from nanovllm.config import Config
+    from nanovllm.models import registry
+    assert registry.architecture_of({"architecture": "Galupel"}) == "Galupel"
+    bad = config([(attn(), None), (attn(kv_heads=1, kv_from=0), None)])        # a reader with other head counts than its source
+    with pytest.raises(AssertionError):
+        from nanovllm import LLM
+        LLM(write_model(tmp_path / "bad", bad, {}), device="cpu", load_format="dummy")
+    with pytest.raises(ValueError):
+        Config(write_model(tmp_path / "bad2", config(DEFAULT, groups=5), {}), device="cpu")       # groups must divide the width
+    # a model without a checkpoint: random tensors under the checkpoint's names go through the same placement
+    from nanovllm import LLM, SamplingParams
+    path = write_model(tmp_path / "dummy", config(DEFAULT), {})
+    llm = LLM(path, device="cpu", dtype=torch.float32, load_format="dummy", max_num_seqs=2, num_kvcache_blocks=4)
+    out = llm.generate([tokens(20, 61, 1)], SamplingParams(max_tokens=3, ignore_eos=True))
+    assert len(out[0]["token_ids"]) == 3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_captured_decode_steps_equal_eager_steps(model, dtype):
+    """Decode-only steps replay a hipGraph per batch-size bucket.  Three requests decode for 70 steps (a block border is
+    crossed, pooled blocks are completed inside replays, the batch shrinks from 3 to 2 to 1: three buckets, padding rows in
+    the bucket of 4) with an eager prefill of a fourth request between replays; every step's logits equal those of an
+    engine that runs everything eagerly."""
+    from nanovllm.engine.llm_engine import LLMEngine
+    from nanovllm.engine.sequence import ACTIVE, Sequence
+    path, cfg, w = model
+    engines = [LLMEngine(path, dtype=dtype, enforce_eager=eager, max_num_seqs=4, num_kvcache_blocks=12, max_model_len=256,
+                         max_num_batched_tokens=4096) for eager in (True, False)]
+    assert not engines[0].model_runner.portion_graphs and sorted(engines[1].model_runner.portion_graphs) == [1, 2, 4]
+    prompts = [tokens(n, cfg["vocab"], 40 + n) for n in (50, 3, 61)]
+    cont = [tokens(70, cfg["vocab"], 50 + i) for i in range(3)]
+    outs = []
+    for eng in engines:
+        seqs, got = [], []
+        for p in prompts:
+            s = Sequence(p)
+            s.state = ACTIVE
+            assert eng.scheduler.reserve_portion(s, len(p))
+            seqs.append(s)
+        got.append(eng.forward_portions([(s, len(s)) for s in seqs]))
+        for s in seqs:
+            s.num_computed = s.num_tokens
+        for step in range(70):
+            live = [(i, s) for i, s in enumerate(seqs) if not (i == 1 and step >= 20) and not (i == 2 and step >= 45)]
+            for i, s in live:
+                s.extend([cont[i][step]])
+                assert eng.scheduler.reserve_portion(s, 1)
+            got.append(eng.forward_portions([(s, 1) for _, s in live]))
+            for _, s in live:
+                s.num_computed += 1
+            if step == 30:                      # eager work between replays: another request's prompt
+                extra = Sequence(tokens(40, cfg["vocab"], 99))
+                extra.state = ACTIVE
+                assert eng.scheduler.reserve_portion(extra, 40)
+                got.append(eng.forward_portions([(extra, 40)]))
+                eng.scheduler.release(extra)
+        outs.append([g.float().cpu() for g in got])
+    assert [a.shape for a in outs[0]] == [b.shape for b in outs[1]]
+    close(torch.cat(outs[1]).numpy(), torch.cat(outs[0]).numpy(), dtype, 0.02)
