@@ -364,4 +364,6 @@ def test_captured_decode_steps_equal_eager_steps(model, dtype):
                 eng.scheduler.release(extra)
         outs.append([g.float().cpu() for g in got])
     assert [a.shape for a in outs[0]] == [b.shape for b in outs[1]]
-    close(torch.cat(outs[1]).numpy(), torch.cat(outs[0]).numpy(), dtype, 0.02)
+    # (float32 is the sharp comparison; in bfloat16 the split count of decode attention differs between the graph's fixed
+    # table width and the eager step's, and that rounding may turn a router's near-tie)
+    close(torch.cat(outs[1]).numpy(), torch.cat(outs[0]).numpy(), dtype, BF16_TIES)
