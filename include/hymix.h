@@ -93,12 +93,12 @@ int hm_attn_rows(int dtype, const void* q, const void* k_cache, const void* v_ca
                  void* o, int64_t T, int H, int G, int D, int V, int block_size, int max_blocks, const void* kp_cache,
                  const void* vp_cache, int pool, int pool_rows, void* stream);
 
-/* For every token of the step whose position ends a block of `pool` tokens: the mean of the block's keys and of its
- * values, as the caches hold them (f32 sums), written to the pooled caches (layout above).  Launch it after the step's
- * keys and values are stored. */
+/* The mean key and mean value of every block of `pool` tokens that the step completes, as the caches hold them (f32
+ * sums), written to the pooled caches (layout above).  Sequence b's portion covers positions [seq_pos0[b], ctx_lens[b]);
+ * max_q = the longest portion of the step.  Launch it after the step's keys and values are stored. */
 int hm_pool_blocks(int dtype, const void* k_cache, const void* v_cache, void* kp_cache, void* vp_cache,
-                   const int32_t* block_tables, const int32_t* tok_seq, const int32_t* tok_pos, int64_t T, int G, int D, int V,
-                   int block_size, int max_blocks, int pool, int pool_rows, void* stream);
+                   const int32_t* block_tables, const int32_t* seq_pos0, const int32_t* ctx_lens, int B, int max_q, int G, int D,
+                   int V, int block_size, int max_blocks, int pool, int pool_rows, void* stream);
 
 /* The same attention on the matrix cores, bf16 storage only, dim and vdim multiples of 8 up to 128, block_size % 64 == 0.
  * Portions of any length (max_q = the longest portion of the step): */

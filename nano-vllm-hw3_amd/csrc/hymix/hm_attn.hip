@@ -205,33 +205,67 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const T* __restrict__ q,
     }
 }
 
-// Mean key and mean value of every block of `pool` tokens that a step completes: one workgroup per token; the token
-// whose position ends a block averages the block's rows as the caches hold them (f32 sums) into the pooled caches.
-template <typename T>
+// Mean key and mean value of every block of `pool` tokens that a step completes.  Sequence b's portion covers the
+// positions [seq_pos0[b], ctx_lens[b]); it completes the blocks seq_pos0[b] / pool .. ctx_lens[b] / pool - 1.  A
+// workgroup owns one such block and kPoolCols packs of VEC channels of the joined [key | value] row; its 256 threads are
+// 8 key lanes x 32 packs: a lane sums every 8th token of the block as the caches hold it (f32), the lanes' partial sums
+// are added in lane order through LDS, so the order of the sum depends on the shapes alone.  (The grid is over blocks,
+// not tokens: the tokens that end a block are a stride apart, which would put all the work on one XCD.)
+constexpr int kPoolChunk = 64;     // tokens whose cache rows are looked up at a time
+constexpr int kPoolCols = 32, kPoolLanes = 8;
+
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void pool_blocks_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                                           T* __restrict__ kp_cache, T* __restrict__ vp_cache,
                                                           const int32_t* __restrict__ block_tables,
-                                                          const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                                                          const int32_t* __restrict__ seq_pos0, const int32_t* __restrict__ ctx_lens,
                                                           int nk, int nv, int block_size, int max_blocks, int pool, int pool_rows) {
-    const int64_t t = blockIdx.x;
-    const int pos = tok_pos[t];
-    if ((pos + 1) % pool != 0) return;
-    const int blk = pos / pool, first = blk * pool;
-    const int32_t* table = block_tables + (size_t)tok_seq[t] * max_blocks;
+    __shared__ float part[kPoolLanes][kPoolCols][VEC];
+    __shared__ int rows[kPoolChunk];
+    const int b = blockIdx.y;
+    const int blk = seq_pos0[b] / pool + blockIdx.x;
+    if (blk >= ctx_lens[b] / pool) return;     // (uniform over the workgroup)
+    const int first = blk * pool;
+    const int32_t* table = block_tables + (size_t)b * max_blocks;
     const size_t prow = (size_t)table[blk / pool_rows] * pool_rows + blk % pool_rows;
     const float inv = 1.f / (float)pool;
-    for (int c = threadIdx.x; c < nk + nv; c += 256) {
-        const bool is_k = c < nk;
-        const T* src = is_k ? k_cache + c : v_cache + (c - nk);
-        const int width = is_k ? nk : nv;
-        float sum = 0.f;
-        for (int j = 0; j < pool; ++j) {
-            const int key = first + j;
-            sum += to_f(src[((size_t)table[key / block_size] * block_size + key % block_size) * width]);
+    struct alignas(sizeof(T) * VEC) Pack { T v[VEC]; };
+    const int tid = threadIdx.x, col = tid % kPoolCols, lane = tid / kPoolCols;
+    const int c = (blockIdx.z * kPoolCols + col) * VEC;          // first channel of this thread's pack: a key channel if c < nk
+    const bool live = c < nk + nv, is_k = c < nk;
+    const T* src = is_k ? k_cache + c : v_cache + (c - nk);
+    const int width = is_k ? nk : nv;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    for (int j0 = 0; j0 < pool; j0 += kPoolChunk) {
+        __syncthreads();                       // the previous chunk's rows are consumed
+        if (tid < kPoolChunk && j0 + tid < pool) {
+            const int key = first + j0 + tid;
+            rows[tid] = table[key / block_size] * block_size + key % block_size;
         }
-        if (is_k) kp_cache[prow * nk + c] = from_f<T>(sum * inv);
-        else vp_cache[prow * nv + (c - nk)] = from_f<T>(sum * inv);
+        __syncthreads();
+        const int n = min(kPoolChunk, pool - j0);
+        if (live)
+            for (int j = lane; j < n; j += kPoolLanes) {
+                const Pack pk = *(const Pack*)(src + (size_t)rows[j] * width);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[e] += to_f(pk.v[e]);
+            }
     }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) part[lane][col][e] = acc[e];
+    __syncthreads();
+    if (!live || lane != 0) return;
+    Pack out;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        float sum = 0.f;
+        for (int l = 0; l < kPoolLanes; ++l) sum += part[l][col][e];
+        out.v[e] = from_f<T>(sum * inv);
+    }
+    if (is_k) *(Pack*)(kp_cache + prow * nk + c) = out;
+    else *(Pack*)(vp_cache + prow * nv + (c - nk)) = out;
 }
 
 }  // namespace hm
@@ -294,19 +328,27 @@ extern "C" int hm_attn_rows(int dtype, const void* q, const void* k_cache, const
 }
 
 extern "C" int hm_pool_blocks(int dtype, const void* k_cache, const void* v_cache, void* kp_cache, void* vp_cache,
-                              const int32_t* block_tables, const int32_t* tok_seq, const int32_t* tok_pos, int64_t T, int G, int D,
-                              int V, int block_size, int max_blocks, int pool, int pool_rows, void* stream) {
-    if (T < 0 || G < 1 || D < 1 || V < 1 || block_size < 1 || max_blocks < 1 || pool < 1 || pool_rows < 1 ||
+                              const int32_t* block_tables, const int32_t* seq_pos0, const int32_t* ctx_lens, int B, int max_q, int G,
+                              int D, int V, int block_size, int max_blocks, int pool, int pool_rows, void* stream) {
+    if (B < 0 || max_q < 0 || G < 1 || D < 1 || V < 1 || block_size < 1 || max_blocks < 1 || pool < 1 || pool_rows < 1 ||
         (int64_t)pool_rows * pool < block_size ||
-        (T > 0 && (!k_cache || !v_cache || !kp_cache || !vp_cache || !block_tables || !tok_seq || !tok_pos))) {
+        (B > 0 && max_q > 0 && (!k_cache || !v_cache || !kp_cache || !vp_cache || !block_tables || !seq_pos0 || !ctx_lens))) {
         set_error("hm_pool_blocks: bad argument");
         return HM_EINVAL;
     }
-    if (T == 0) return HM_OK;
-    HM_DISPATCH(dtype, "hm_pool_blocks",
-                hipLaunchKernelGGL(pool_blocks_kernel<DT>, dim3((unsigned)T), dim3(256), 0, as_stream(stream), (const DT*)k_cache,
-                                   (const DT*)v_cache, (DT*)kp_cache, (DT*)vp_cache, block_tables, tok_seq, tok_pos, G * D, G * V,
-                                   block_size, max_blocks, pool, pool_rows));
+    if (B > 65535) { set_error("hm_pool_blocks: at most 65535 sequences"); return HM_ESHAPE; }
+    if (B == 0 || max_q == 0) return HM_OK;
+    // packs of 8 channels (16 bytes in bf16) when every row starts and ends on a multiple of 8
+    const bool wide = (G * D) % 8 == 0 && (G * V) % 8 == 0;
+    const uintptr_t bits = (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)kp_cache | (uintptr_t)vp_cache;
+    const int blocks = max_q / pool + 1;       // the most blocks a portion of max_q tokens completes
+#define HM_POOL(VEC_)                                                                                                      \
+    hipLaunchKernelGGL((pool_blocks_kernel<DT, VEC_>),                                                                    \
+                       dim3((unsigned)blocks, (unsigned)B, (unsigned)((G * (D + V) / VEC_ + kPoolCols - 1) / kPoolCols)),  \
+                       dim3(256), 0, as_stream(stream), (const DT*)k_cache, (const DT*)v_cache, (DT*)kp_cache, (DT*)vp_cache, \
+                       block_tables, seq_pos0, ctx_lens, G * D, G * V, block_size, max_blocks, pool, pool_rows)
+    HM_DISPATCH(dtype, "hm_pool_blocks", if (wide && bits % (8 * sizeof(DT)) == 0) HM_POOL(8); else HM_POOL(1));
+#undef HM_POOL
     HM_CHECK_LAUNCH("hm_pool_blocks");
     return HM_OK;
 }

@@ -27,7 +27,7 @@ SIGNATURES = {
                               _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp]),
     "hm_attn_rows": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _f, _vp, _i64, _int, _int, _int, _int, _int,
                             _int, _vp, _vp, _int, _int, _vp]),
-    "hm_pool_blocks": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _int, _int, _int, _int, _vp]),
+    "hm_pool_blocks": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _int, _int, _int, _vp]),
     "hm_attn_tiles": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _f, _vp, _int, _int, _int, _int, _int, _int, _int, _int,
                              _vp, _vp, _int, _int, _vp]),
     "hm_attn_decode_workspace_bytes": (_sz, [_i64, _int, _int, _int]),

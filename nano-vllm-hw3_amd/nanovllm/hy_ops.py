@@ -127,17 +127,17 @@ def pool_rows_per_page(block_size, pool):
 
 
 def pool_blocks(k_cache, v_cache, kp_cache, vp_cache, pool, ctx: StepContext):
-    """For every token of the step whose position ends a block of ``pool`` tokens: the block's mean key and mean value, as
-    the caches hold them, into the pooled caches [blocks, pool_rows_per_page, G, D | V].  Call it after the step's keys
+    """For every block of ``pool`` tokens that the step completes: the block's mean key and mean value, as the caches hold
+    them, into the pooled caches [blocks, pool_rows_per_page, G, D | V].  Call it after the step's keys
     and values are stored."""
     if not k_cache.is_cuda:
         return cpu_ops.pool_blocks(k_cache, v_cache, kp_cache, vp_cache, pool, ctx)
     bs, G, D, V = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3], v_cache.shape[3]
     assert kp_cache.shape[1] == vp_cache.shape[1] == pool_rows_per_page(bs, pool) and kp_cache.dtype == k_cache.dtype
     HM.check(HM.load().hm_pool_blocks(HM.dtype_code(k_cache.dtype), k_cache.data_ptr(), v_cache.data_ptr(), kp_cache.data_ptr(),
-                                      vp_cache.data_ptr(), ctx.block_tables.data_ptr(), ctx.tok_seq.data_ptr(),
-                                      ctx.tok_pos.data_ptr(), ctx.num_tokens, G, D, V, bs, ctx.block_tables.shape[1], int(pool),
-                                      kp_cache.shape[1], _dev(k_cache)))
+                                      vp_cache.data_ptr(), ctx.block_tables.data_ptr(), ctx.seq_pos0.data_ptr(),
+                                      ctx.ctx_lens.data_ptr(), ctx.num_seqs, int(ctx.max_q), G, D, V, bs, ctx.block_tables.shape[1],
+                                      int(pool), kp_cache.shape[1], _dev(k_cache)))
 
 
 USE_TILES = True       # bf16 attention on the matrix cores where the shape allows (tests compare both forms)

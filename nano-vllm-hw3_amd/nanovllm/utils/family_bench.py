@@ -1,6 +1,8 @@
 """Throughput of the Pasizen or the Lipelix family beside the Qwen3 decoder at equal size (random weights, bf16, one
 GPU), and the time of every libseqmix / libhymix kernel beside the like kernel of the Qwen3 path with both against their
-rooflines.  Used by ``bench.py --families [--family NAME]``; prints one JSON object."""
+rooflines; for the Galupel family the comparison is with Pasizen, the closest of the three (latent attention and routed
+experts), and its kernels stand beside the forms of the same kernels that Pasizen and Lipelix run.  Used by
+``bench.py --families [--family NAME]``; prints one JSON object."""
 import json
 import os
 import tempfile
@@ -50,6 +52,25 @@ def lipelix_config(width, heads, ff, layers):
                 layers=[dict(type=kinds[i % 4][0], mixer=kinds[i % 4][1], mlp=dict(kind="dense", ff=ff)) for i in range(layers)])
 
 
+def galupel_config(width, heads, ff, layers, rank):
+    """Latent attention (a 64-channel rotated part beside the latent, so that a cache row is as wide as Pasizen's at the
+    size; 512-token window) and grouped-head attention (heads / 2 key/value heads of 128, 512-token window, pooled blocks
+    of 64 tokens) alternate; every second attention layer reads the keys and values of the one before it; every layer has
+    16 GELU experts of ff/4 with 4 chosen (best 2 of 4 groups): the active feed-forward width is ff."""
+    lat = dict(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=rank - 64, scale=192 ** -0.5, rot=dict(dims=64, base=10000.0),
+               mask=dict(size=512))
+    att = dict(heads=heads, kv_heads=max(1, heads // 2), dim=128, vdim=128, scale=128 ** -0.5, mask=dict(size=512, pool=64))
+    moe = dict(kind="moe", expert=dict(ff=ff // 4), router=dict(experts=16, top=4, groups=dict(count=4, keep=2)))
+    specs = []
+    for i in range(layers):
+        if i % 2 == 0:
+            specs.append(dict(type="latent_attention", mixer=lat, mlp=moe))
+        else:
+            specs.append(dict(type="attention", mixer=dict(att, kv_from=i - 2) if i % 4 == 3 else att, mlp=moe))
+    return dict(architecture="Galupel", vocab=VOCAB, width=width, norm=dict(eps=1e-5, groups=4), logit_scale=1.0, logit_softcap=30.0,
+                max_positions=8192, layers=specs)
+
+
 def _model_dir(cfg):
     d = tempfile.mkdtemp(prefix="family_bench_")
     with open(os.path.join(d, "config.json"), "w") as f:
@@ -74,7 +95,8 @@ def engine_throughput(family, size, prefill_seqs=8, prefill_len=1024, decode_seq
     from nanovllm.engine.sequence import ACTIVE, Sequence
     width, heads, ff, layers, rank = SIZES[size]
     cfg = (pasizen_config(width, heads, ff, layers, rank) if family == "pasizen" else
-           lipelix_config(width, heads, ff, layers) if family == "lipelix" else qwen3_config(width, heads, ff, layers))
+           lipelix_config(width, heads, ff, layers) if family == "lipelix" else
+           galupel_config(width, heads, ff, layers, rank) if family == "galupel" else qwen3_config(width, heads, ff, layers))
     llm = LLM(_model_dir(cfg), load_format="dummy", enforce_eager=False, max_model_len=2048,
               max_num_seqs=decode_seqs, max_num_batched_tokens=prefill_seqs * prefill_len, gpu_memory_utilization=0.5)
     g = torch.Generator().manual_seed(0)
@@ -375,11 +397,142 @@ def hymix_kernel_table(width=2048, heads=16, ff=6144, T=8192, seq=1024, B=64, ct
     return rows
 
 
+def galupel_kernel_table(width=2048, heads=16, rank=256, ff=6144, T=8192, seq=1024, B=64, ctx=1024, window=512, pool=64):
+    """Seconds per launch of every kernel form the Galupel family runs at a layer's size, its bound and the fraction of it
+    reached; beside each the form of the same kernel that the closest existing family runs (`like`)."""
+    from nanovllm import hy_ops, seq_ops
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def add(name, like, sec, bytes_=0, flops=0):
+        bound = max(bytes_ / (HBM_GBPS * 1e9), flops / (MFMA_TFLOPS * 1e12))
+        rows.append(dict(kernel=name, like=like, us=round(sec * 1e6, 1), bound_us=round(bound * 1e6, 1),
+                         of_roofline=round(bound / sec, 3), bound="flops" if flops / (MFMA_TFLOPS * 1e12) > bytes_ / (HBM_GBPS * 1e9) else "bytes"))
+    r = lambda *s: torch.randn(*s, device=dev).to(bf)  # noqa: E731
+    nseq, bs, G, D, Rd = T // seq, 64, heads // 2, 128, 64
+    R = rank - Rd
+    import numpy as np
+
+    def context(portions):
+        tables, nxt = [], 0
+        for p0, n in portions:
+            nb = (p0 + n + bs - 1) // bs
+            tables.append(list(range(nxt, nxt + nb)))
+            nxt += nb
+        tok_seq = np.concatenate([np.full(n, b) for b, (_, n) in enumerate(portions)])
+        tok_pos = np.concatenate([np.arange(p0, p0 + n) for p0, n in portions])
+        slot = np.concatenate([np.asarray(tables[b])[np.arange(p0, p0 + n) // bs] * bs + np.arange(p0, p0 + n) % bs
+                               for b, (p0, n) in enumerate(portions)])
+        mb = max(len(t) for t in tables)
+        bt = np.zeros((len(portions), mb), dtype=np.int32)
+        for b, t in enumerate(tables):
+            bt[b, :len(t)] = t
+        qs = np.concatenate([[0], np.cumsum([n for _, n in portions])])
+        i32 = lambda v: torch.tensor(np.asarray(v), dtype=torch.int32, device=dev)  # noqa: E731
+        return seq_ops.StepContext(tok_seq=i32(tok_seq), tok_pos=i32(tok_pos), qstart=i32(qs), seq_pos0=i32([p for p, _ in portions]),
+                                   ctx_lens=i32([p + n for p, n in portions]), seq_slot=i32(list(range(len(portions)))),
+                                   slot_mapping=i32(slot), block_tables=i32(bt), num_seqs=len(portions), num_tokens=int(qs[-1]),
+                                   max_q=max(n for _, n in portions), block_size=bs, qstart_host=qs.tolist()), nxt
+    pre, nblk_p = context([(0, seq)] * nseq)
+    dec, nblk_d = context([(ctx - 1, 1)] * B)
+    nblk = max(nblk_p, nblk_d)
+    # ---- residual boundary: grouped norm of the result + add + the reader's copy | Pasizen: stream step, Lipelix: gated close
+    x, y, pw, nw = torch.randn(T, width, device=dev), r(T, width), r(width), r(width)
+    add("hm_group_norm_residual (T=%d)" % T, "hm_sublayer_close", _event_time(lambda: hy_ops.group_norm_residual(x, y, pw, 4, 1e-5, bf)),
+        bytes_=T * width * (8 + 2 + 2))
+    gate, gb = r(T, width), r(width)
+    add("hm_sublayer_close (T=%d)" % T, "-", _event_time(lambda: hy_ops.sublayer_close(x, y, gate, gb, pw, 0.5, nw, 1e-5, bf)),
+        bytes_=T * width * (8 + 2 + 2 + 2))
+    # ---- q/k/v preparation: per-head norm with a shared weight row, per-head temperature | Lipelix: unit-norm heads + rotation
+    kc, vc = r(nblk, bs, G, D), r(nblk, bs, G, D)
+    qkv = r(T, (heads + 2 * G) * D)
+    hw, temp = r(D), torch.rand(heads, device=dev) + 0.5
+    add("hm_qkv_prepare (T=%d, head norm + temperature)" % T, "hm_qkv_prepare (unit norm)",
+        _event_time(lambda: hy_ops.qkv_prepare(qkv, heads, G, D, D, None, None, 1e-5, None, False, pre, kc, vc, None, None, hw, hw, temp)),
+        bytes_=T * (heads + 2 * G) * D * 4)
+    inv_freq = hy_ops.rotary_inv_freq(64, 1e4, dev)
+    add("hm_qkv_prepare (T=%d, unit norm)" % T, "-",
+        _event_time(lambda: hy_ops.qkv_prepare(qkv, heads, G, D, D, None, None, 1e-5, inv_freq, True, pre, kc, vc, None, None)),
+        bytes_=T * (heads + 2 * G) * D * 4)
+    pr = hy_ops.pool_rows_per_page(bs, pool)
+    kp, vp = r(nblk, pr, G, D), r(nblk, pr, G, D)
+    add("hm_pool_blocks (T=%d, pool %d)" % (T, pool), "-", _event_time(lambda: hy_ops.pool_blocks(kc, vc, kp, vp, pool, pre)),
+        bytes_=T * G * D * 4 + T // pool * G * D * 4)
+    # ---- attention, prefill: window + pooled blocks | Lipelix: window + kept first tokens
+    q = r(T, heads, D)
+    wpairs = nseq * heads * sum(min(i + 1, window) + max(0, (i + 1 - window) // pool) for i in range(seq))
+    add("hm_attn_tiles window %d + pooled %d (%dx%d)" % (window, pool, nseq, seq), "hm_attn_tiles window",
+        _event_time(lambda: hy_ops.paged_attention(q, kc, vc, pre, 0.09, None, window, 0, pooled=(kp, vp, pool)), 5), flops=wpairs * 4 * D)
+    sink = torch.randn(heads, device=dev)
+    kpairs = nseq * heads * sum(min(i + 1, window) + min(4, max(0, i + 1 - window)) for i in range(seq))
+    add("hm_attn_tiles window %d+4 kept (%dx%d)" % (window, nseq, seq), "-",
+        _event_time(lambda: hy_ops.paged_attention(q, kc, vc, pre, 0.09, sink, window, 4), 5), flops=kpairs * 4 * D)
+    # ---- attention, decode
+    qd = r(B, heads, D)
+    seen = max(0, (ctx - window) // pool)
+    add("hm_attn_decode window %d + pooled %d (B=%d, ctx=%d)" % (window, pool, B, ctx), "hm_attn_decode window",
+        _event_time(lambda: hy_ops.paged_attention(qd, kc, vc, dec, 0.09, None, window, 0, pooled=(kp, vp, pool))),
+        bytes_=B * (window + seen) * G * D * 4)
+    add("hm_attn_decode window %d+4 kept (B=%d, ctx=%d)" % (window, B, ctx), "-",
+        _event_time(lambda: hy_ops.paged_attention(qd, kc, vc, dec, 0.09, sink, window, 4)), bytes_=B * (window + 4) * G * D * 4)
+    # ---- latent side: norm + rotation + store | Pasizen: norm + store
+    cache = r(nblk, bs, rank)
+    qc = r(T, heads * (D + Rd) + rank)
+    qa = r(T, heads, rank)
+    lw = r(R)
+    nq = heads * (D + Rd)
+    add("sm_latent_rope_store (T=%d, H=%d)" % (T, heads), "sm_latent_norm_store",
+        _event_time(lambda: seq_ops.latent_rope_store(qc[:, nq:], lw, 1e-5, qc[:, :nq], qa, inv_freq, Rd, heads, D, R, Rd, cache, pre)),
+        bytes_=T * (rank * 4 + heads * Rd * 4))
+    add("sm_latent_norm_store (T=%d)" % T, "-",
+        _event_time(lambda: seq_ops.latent_norm_store(qc[:, nq:], nw[:rank].contiguous(), 1e-5, cache, pre.slot_mapping)), bytes_=T * rank * 4)
+    lpairs = nseq * heads * sum(min(i + 1, window) for i in range(seq))
+    add("sm_latent_attn_tiles window %d, row %d+%d (%dx%d, H=%d)" % (window, R, Rd, nseq, seq, heads), "sm_latent_attn_tiles",
+        _event_time(lambda: seq_ops.latent_attention(qa, cache, pre, 0.09, value_cols=R, window=window), 5), flops=lpairs * 2 * (rank + R))
+    pairs = nseq * seq * (seq + 1) / 2 * heads
+    add("sm_latent_attn_tiles full, row %d (%dx%d, H=%d)" % (rank, nseq, seq, heads), "-",
+        _event_time(lambda: seq_ops.latent_attention(qa, cache, pre, 0.09), 5), flops=pairs * 4 * rank)
+    qad = r(B, heads, rank)
+    add("sm_latent_attn_decode window %d, row %d+%d (B=%d, ctx=%d)" % (window, R, Rd, B, ctx), "sm_latent_attn_decode",
+        _event_time(lambda: seq_ops.latent_attention(qad, cache, dec, 0.09, value_cols=R, window=window)), bytes_=B * window * rank * 2)
+    add("sm_latent_attn_decode full, row %d (B=%d, ctx=%d)" % (rank, B, ctx), "-",
+        _event_time(lambda: seq_ops.latent_attention(qad, cache, dec, 0.09)), bytes_=B * ctx * rank * 2)
+    # ---- router and experts: sigmoid + correction + no renormalisation, GELU experts | Pasizen: softmax, clamped GLU
+    E, top, F = 16, 4, ff // 4
+    h = r(T, width)
+    rw, corr = torch.randn(E, width, device=dev), torch.randn(E, device=dev) * 0.1
+    add("sm_moe_route sigmoid + correction (T=%d, E=%d)" % (T, E), "sm_moe_route softmax",
+        _event_time(lambda: seq_ops.moe_route(h, rw, top, 4, 2, seq_ops.ROUTE_SIGMOID, corr, 2, False)), bytes_=T * width * 2)
+    add("sm_moe_route softmax (T=%d, E=%d)" % (T, E), "-", _event_time(lambda: seq_ops.moe_route(h, rw, top, 4, 2)), bytes_=T * width * 2)
+    idx, wts = seq_ops.moe_route(h, rw, top, 4, 2, seq_ops.ROUTE_SIGMOID, corr, 2, False)
+    w_up, w_gu, w_down = r(E, F, width), r(E, 2 * F, width), r(E, width, F)
+    t_gelu = (seq_ops.tile_expert_weights(w_up, 1), seq_ops.tile_expert_weights(w_down))
+    t_glu = (seq_ops.tile_expert_weights(w_gu, 2), t_gelu[1])
+    add("sm_moe_tiles128 GELU experts (T=%d, top %d of %d, F=%d)" % (T, top, E, F), "sm_moe_tiles128 clamped GLU",
+        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_up, w_down, 0.0, form="tiles128", tiled=t_gelu, act_kind=seq_ops.ACT_GELU), 5),
+        flops=T * top * 4 * width * F)
+    add("sm_moe_tiles128 clamped GLU (T=%d)" % T, "-",
+        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_gu, w_down, 7.0, form="tiles128", tiled=t_glu), 5), flops=T * top * 6 * width * F)
+    hd = h[:B].contiguous()
+    idx_d, wts_d = seq_ops.moe_route(hd, rw, top, 4, 2, seq_ops.ROUTE_SIGMOID, corr, 2, False)
+    touched = len(torch.unique(idx_d))
+    add("sm_moe_grouped GELU experts (T=%d: decode)" % B, "sm_moe_grouped clamped GLU",
+        _event_time(lambda: seq_ops.moe_experts(hd, idx_d, wts_d, w_up, w_down, 0.0, form="grouped", tiled=t_gelu, act_kind=seq_ops.ACT_GELU)),
+        bytes_=touched * 2 * F * width * 2)
+    add("sm_moe_grouped clamped GLU (T=%d: decode)" % B, "-",
+        _event_time(lambda: seq_ops.moe_experts(hd, idx_d, wts_d, w_gu, w_down, 7.0, form="grouped", tiled=t_glu)),
+        bytes_=touched * 3 * F * width * 2)
+    lg = torch.randn(B, VOCAB, device=dev)
+    add("hm_scale_softcap (B=%d, vocab %d)" % (B, VOCAB), "-", _event_time(lambda: hy_ops.scale_softcap_(lg, 1.0, 30.0)), bytes_=B * VOCAB * 8)
+    return rows
+
+
 def main(sizes=("w1024", "w2048"), kernels=True, family="pasizen"):
     out = dict(metric="family comparison", dtype="bf16", data="synthetic (random weights)", throughput=[], kernels=[])
     for size in sizes:
-        for fam in (family, "qwen3"):
+        for fam in ((family, "pasizen", "qwen3") if family == "galupel" else (family, "qwen3")):
             out["throughput"].append(engine_throughput(fam, size))
     if kernels:
-        out["kernels"] = kernel_table() if family == "pasizen" else hymix_kernel_table()
+        out["kernels"] = (kernel_table() if family == "pasizen" else galupel_kernel_table() if family == "galupel" else
+                          hymix_kernel_table())
     return out
