@@ -13,23 +13,52 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, const float* __restrict__ router_w,
                                                         int32_t* __restrict__ idx, float* __restrict__ wts, int64_t T_all, int W,
                                                         int E, int top, int groups, int keep, int score,
-                                                        const float* __restrict__ correction, int group_top, int renorm) {
-    extern __shared__ float z_all[];             // per token: E scores, then `groups` group scores
+                                                        const float* __restrict__ correction, int group_top, int renorm,
+                                                        int staged) {
+    extern __shared__ float z_all[];             // per token: E scores, then `groups` group scores; then the staged rows
     const int64_t t0 = (int64_t)blockIdx.x * kRouteTokens;
     const int nt = (int)min((int64_t)kRouteTokens, T_all - t0);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int e = wave; e < E; e += 4) {
-        const float* wr = router_w + (size_t)e * W;
-        float d[kRouteTokens];
-        for (int i = 0; i < kRouteTokens; ++i) d[i] = 0.f;
-        for (int c = lane; c < W; c += 64) {
-            const float wv = wr[c];
-            for (int i = 0; i < kRouteTokens; ++i)
-                if (i < nt) d[i] += to_f(h[(size_t)(t0 + i) * W + c]) * wv;
+    if (staged) {
+        // the workgroup's token rows (one contiguous piece of h) go to LDS once; every expert's row is then read once per
+        // workgroup in 16-byte pieces and meets all the tokens there
+        T* h_lds = (T*)(z_all + kRouteTokens * (E + groups));
+        const T* src = h + (size_t)t0 * W;
+        struct alignas(sizeof(T) * 4) Pack4 { T v[4]; };
+        for (int i = threadIdx.x * 4; i < nt * W; i += 1024) *(Pack4*)(h_lds + i) = *(const Pack4*)(src + i);     // W % 4 == 0
+        __syncthreads();
+        for (int e = wave; e < E; e += 4) {
+            const float* wr = router_w + (size_t)e * W;
+            float d[kRouteTokens];
+            for (int i = 0; i < kRouteTokens; ++i) d[i] = 0.f;
+            for (int c = lane * 4; c < W; c += 256) {
+                const float4 wv = *(const float4*)(wr + c);
+#pragma unroll
+                for (int i = 0; i < kRouteTokens; ++i)
+                    if (i < nt) {
+                        const Pack4 hv = *(const Pack4*)(h_lds + (size_t)i * W + c);
+                        d[i] += to_f(hv.v[0]) * wv.x + to_f(hv.v[1]) * wv.y + to_f(hv.v[2]) * wv.z + to_f(hv.v[3]) * wv.w;
+                    }
+            }
+            for (int i = 0; i < kRouteTokens; ++i) {
+                const float sum = wave_sum(d[i]);
+                if (lane == 0) z_all[i * (E + groups) + e] = sum;
+            }
         }
-        for (int i = 0; i < kRouteTokens; ++i) {
-            const float s = wave_sum(d[i]);
-            if (lane == 0) z_all[i * (E + groups) + e] = s;
+    } else {
+        for (int e = wave; e < E; e += 4) {
+            const float* wr = router_w + (size_t)e * W;
+            float d[kRouteTokens];
+            for (int i = 0; i < kRouteTokens; ++i) d[i] = 0.f;
+            for (int c = lane; c < W; c += 64) {
+                const float wv = wr[c];
+                for (int i = 0; i < kRouteTokens; ++i)
+                    if (i < nt) d[i] += to_f(h[(size_t)(t0 + i) * W + c]) * wv;
+            }
+            for (int i = 0; i < kRouteTokens; ++i) {
+                const float sum = wave_sum(d[i]);
+                if (lane == 0) z_all[i * (E + groups) + e] = sum;
+            }
         }
     }
     __syncthreads();
@@ -191,19 +220,27 @@ __global__ __launch_bounds__(256) void moe_pairs_gate_up_kernel(const T* __restr
 template <typename T>
 __global__ __launch_bounds__(256) void moe_pairs_down_kernel(const T* __restrict__ act, const int32_t* __restrict__ idx,
                                                              const float* __restrict__ wts, const T* __restrict__ w_down,
-                                                             const T* __restrict__ shared, T* __restrict__ y, int top, int W, int F) {
-    extern __shared__ float a_lds[];             // top * F activations of the token's pairs
+                                                             const T* __restrict__ shared, T* __restrict__ y, int top, int W, int F,
+                                                             int staged) {
+    extern __shared__ float a_lds[];             // top * F activations of the token's pairs (staged: they fit)
     const int64_t t = blockIdx.x;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int c = threadIdx.x; c < top * F; c += 256) a_lds[c] = to_f(act[(size_t)t * top * F + c]);
-    __syncthreads();
+    if (staged) {
+        for (int c = threadIdx.x; c < top * F; c += 256) a_lds[c] = to_f(act[(size_t)t * top * F + c]);
+        __syncthreads();
+    }
+    const T* a_row = act + (size_t)t * top * F;
     for (int w = wave; w < W; w += 4) {
         float tot = 0.f;
         for (int k = 0; k < top; ++k) {
             const int e = idx[(size_t)t * top + k];
             const T* row = w_down + ((size_t)e * W + w) * F;
             float d = 0.f;
-            for (int c = lane; c < F; c += 64) d += a_lds[k * F + c] * to_f(row[c]);
+            if (staged) {
+                for (int c = lane; c < F; c += 64) d += a_lds[k * F + c] * to_f(row[c]);
+            } else {                                 // the same sum from global memory
+                for (int c = lane; c < F; c += 64) d += to_f(a_row[k * F + c]) * to_f(row[c]);
+            }
             d = wave_sum(d);
             tot += wts[(size_t)t * top + k] * to_f(from_f<T>(d));
         }
@@ -232,10 +269,14 @@ extern "C" int sm_moe_route(int dtype, const void* h, const float* router_w, int
         return SM_ESHAPE;
     }
     if (T == 0) return SM_OK;
+    // the token rows of a workgroup are staged in LDS when they fit and the rows can be moved in pieces of four channels
+    const size_t scores = (size_t)kRouteTokens * (E + groups) * 4;
+    const size_t rows = (size_t)kRouteTokens * W * (dtype == SM_F32 ? 4 : 2);
+    const int staged = W % 4 == 0 && scores % 16 == 0 && scores + rows <= 60 * 1024 && ((uintptr_t)h | (uintptr_t)router_w) % 16 == 0;
     SM_DISPATCH(dtype, "sm_moe_route",
                 hipLaunchKernelGGL(moe_route_kernel<DT>, dim3((unsigned)((T + kRouteTokens - 1) / kRouteTokens)), dim3(256),
-                                   (size_t)kRouteTokens * (E + groups) * 4, as_stream(stream), (const DT*)h, router_w, idx, wts, T, W, E,
-                                   top, groups, keep, score, correction, group_top, renorm));
+                                   scores + (staged ? rows : 0), as_stream(stream), (const DT*)h, router_w, idx, wts, T, W, E,
+                                   top, groups, keep, score, correction, group_top, renorm, staged));
     SM_CHECK_LAUNCH("sm_moe_route");
     return SM_OK;
 }
@@ -261,11 +302,12 @@ extern "C" int sm_moe_pairs_down(int dtype, const void* act, const int32_t* idx,
         set_error("sm_moe_pairs_down: bad argument");
         return SM_EINVAL;
     }
-    if ((size_t)top * F * 4 > 60000) { set_error("sm_moe_pairs_down: top * F too large"); return SM_ESHAPE; }
     if (T == 0) return SM_OK;
+    const int staged = (size_t)top * F * 4 <= 60000;            // a token's activations in LDS when they fit
     SM_DISPATCH(dtype, "sm_moe_pairs_down",
-                hipLaunchKernelGGL(moe_pairs_down_kernel<DT>, dim3((unsigned)T), dim3(256), (size_t)top * F * 4, as_stream(stream),
-                                   (const DT*)act, idx, wts, (const DT*)w_down, (const DT*)shared, (DT*)y, top, W, F));
+                hipLaunchKernelGGL(moe_pairs_down_kernel<DT>, dim3((unsigned)T), dim3(256), staged ? (size_t)top * F * 4 : 0,
+                                   as_stream(stream), (const DT*)act, idx, wts, (const DT*)w_down, (const DT*)shared, (DT*)y, top, W,
+                                   F, staged));
     SM_CHECK_LAUNCH("sm_moe_pairs_down");
     return SM_OK;
 }

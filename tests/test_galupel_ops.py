@@ -281,7 +281,7 @@ def test_sigmoid_router_with_correction(device, dtype, E, top, groups, keep):
 
 @pytest.mark.parametrize("device,dtype", CASES)
 @pytest.mark.parametrize("form", [None, "pairs", "grouped", "tiles128"])
-@pytest.mark.parametrize("E,top,W,F,T", [(6, 2, 32, 24, 19), (4, 4, 72, 8, 150), (3, 1, 40, 136, 5)])
+@pytest.mark.parametrize("E,top,W,F,T", [(6, 2, 32, 24, 19), (4, 4, 72, 8, 150), (3, 1, 40, 136, 5), (2, 2, 16, 7608, 3)])
 def test_gelu_experts(device, dtype, form, E, top, W, F, T):
     if form in ("grouped", "tiles128") and (device == "cpu" or dtype != torch.bfloat16):
         pytest.skip("the matrix-core forms are bfloat16 kernels")
