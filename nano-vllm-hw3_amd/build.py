@@ -3,9 +3,11 @@
 Three libraries, each from its own folder of translation units, so that a model only waits for what it runs on:
   qlinear  csrc/*.hip         -> nanovllm/_lib/libqlinear.so   (quantized linears, Qwen3 operators, attention)
   seqmix   csrc/seqmix/*.hip  -> nanovllm/_lib/libseqmix.so    (multi-stream residuals, short convolutions, latent
-                                                                attention, PolyNorm / clamped GLU, expert routing)
-  hymix    csrc/hymix/*.hip   -> nanovllm/_lib/libhymix.so     (gated residual, token shift, rotary attention with sinks
-                                                                and windows over a paged cache, delta-rule recurrence)
+                                                                attention with or without a rotated part and a window,
+                                                                PolyNorm / clamped GLU / GELU experts, expert routing)
+  hymix    csrc/hymix/*.hip   -> nanovllm/_lib/libhymix.so     (gated and grouped-norm residuals, token shift, attention
+                                                                with sinks, windows and pooled blocks over a paged
+                                                                cache, delta-rule recurrence)
 ``python build.py [--force] [qlinear|seqmix|hymix]`` builds one of them, or all without a name."""
 import os
 import shutil

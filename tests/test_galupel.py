@@ -244,6 +244,57 @@ def test_other_shapes(tmp_path, device, name):
         close(allg, allr, dtype, BF16_TIES)
 
 
+def random_config(seed):
+    """A configuration drawn from the design's whole space: width, norm groups, 1-6 layers of either mixer in any order,
+    head counts and sizes on and off the matrix-core tiles, windows and pooled blocks around and beyond a cache block,
+    readers of earlier layers' keys and values, layers without a feed-forward, routers with 1-4 groups of 1-4 experts."""
+    import random
+    r = random.Random(seed)
+    width = r.choice([32, 48, 64, 96, 136])
+    groups = r.choice([g for g in (1, 2, 4, 8, 17) if width % g == 0])
+    layers, sources = [], {}
+    for i in range(r.randint(1, 6)):
+        mlp = None
+        if r.random() < 0.75:
+            count, per = r.choice([1, 2, 3, 4]), r.choice([1, 2, 3, 4])
+            keep = r.randint(1, count)
+            mlp = moe(experts=count * per, top=r.randint(1, min(keep * per, 6)), ff=r.choice([8, 16, 24, 40]), groups=(count, keep))
+        if r.random() < 0.5:
+            kvh, rep = r.choice([1, 2, 4]), r.choice([1, 2, 4])
+            dim, vdim = r.choice([8, 16, 32, 64, 20]), r.choice([8, 16, 32, 64, 12])
+            src = sources.get((kvh, dim, vdim)) if r.random() < 0.7 else None
+            layers.append((attn(heads=kvh * rep, kv_heads=kvh, dim=dim, vdim=vdim, scale=dim ** -0.5 * r.choice([1.0, 2.0]),
+                                window=r.choice([1, 2, 7, 16, 40, 64, 100, 130]), pool=r.choice([1, 2, 5, 11, 16, 64, 80]), kv_from=src), mlp))
+            if src is None:
+                sources[(kvh, dim, vdim)] = i
+        else:
+            layers.append((latent(heads=r.choice([1, 2, 3, 4, 8]), dim=r.choice([4, 8, 16, 32]), rot_dim=r.choice([2, 4, 8, 16, 32]),
+                                  vdim=r.choice([4, 8, 16, 32]), kv_rank=r.choice([8, 16, 24, 64, 96, 36]), scale=0.2,
+                                  window=r.choice([1, 3, 30, 64, 65, 130, 500]), base=r.choice([50.0, 10000.0])), mlp))
+    return config(layers, width=width, vocab=r.choice([37, 64, 200]), groups=groups, logit_scale=r.choice([0.5, 1.0, 2.0]),
+                  softcap=r.choice([0.0, 10.0, 30.0]))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("seed", range(6))
+def test_random_configurations(tmp_path, device, seed):
+    """Configurations drawn at random, in float32 (the sharp comparison; bfloat16 is bounded per mechanism and on the
+    fixed configurations): a prompt in two portions, a second request beside it, then single tokens."""
+    cfg = random_config(seed)
+    w = weights(cfg, seed=seed)
+    path = write_model(tmp_path / "m", cfg, w)
+    n = 150
+    a, b = tokens(n, cfg["vocab"], seed), tokens(40, cfg["vocab"], seed + 100)
+    ra, rb = forward(cfg, w, a), forward(cfg, w, b)
+    c1 = 1 + (seed * 37) % (n - 40)
+    steps = [([("a", a[:c1], list(range(c1)))], []),
+             ([("a", a[c1:n - 20], list(range(n - 20 - c1))), ("b", b[:7], list(range(7)))], []),
+             ([("b", b[7:], list(range(33))), ("a", a[n - 20:n - 19], [0])], ["b"])] + [([("a", [t], [0])], []) for t in a[n - 19:]]
+    got = replay(path, steps, tmp_path, device, torch.float32, max_tokens=256)
+    close(np.concatenate([got[i] for i in range(len(steps))]),
+          np.concatenate([ra[:c1], ra[c1:n - 20], rb[:7], rb[7:], ra[n - 20:n - 19], ra[n - 19:]]), torch.float32)
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_far_blocks_and_window_edges_show(tmp_path, device):
     """Weights made so that faults show: a token's key is its first head's query and the scores are steep, so equal tokens
