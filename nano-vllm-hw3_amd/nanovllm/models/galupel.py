@@ -41,9 +41,13 @@ class GalupelLayer(nn.Module):
             src = m.get("kv_from")
             if src is not None and not (0 <= src < len(earlier) and isinstance(earlier[src].mixer, PagedRotaryAttention)):
                 raise ValueError(f"kv_from: {src} is not an earlier attention layer")
-            self.mixer = PagedRotaryAttention(W, m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"], eps, 0, 1.0,
+            source = earlier[src].mixer if src is not None else None
+            # a reader's key/value head count and value size are its source's (config.json may repeat them)
+            kv_heads = m["kv_heads"] if "kv_heads" in m or source is None else source.kv_heads
+            vdim = m["vdim"] if "vdim" in m or source is None else source.vdim
+            self.mixer = PagedRotaryAttention(W, m["heads"], kv_heads, m["dim"], vdim, m["scale"], eps, 0, 1.0,
                                               window=mask.get("size", 0), pool=mask.get("pool", 0), head_norm=True,
-                                              head_temp=True, kv_source=earlier[src].mixer if src is not None else None)
+                                              head_temp=True, kv_source=source)
         elif self.kind == "latent_attention":
             rot = m.get("rot") or {}
             self.mixer = LatentAttention(W, m["heads"], m["dim"], m["vdim"], m["kv_rank"], m["scale"], eps,
@@ -156,7 +160,7 @@ class GalupelForCausalLM(nn.Module):
             t[p + "norm1"] = 0.5 + rnd(W)
             H, D, V = m["heads"], m["dim"], m["vdim"]
             if spec["type"] == "attention":
-                G = m["kv_heads"]
+                G = m.get("kv_heads", 1)                       # (not needed by a layer that reads another layer's)
                 t.update({p + "mix.q": rnd(H * D, W, s=W ** -0.5), p + "mix.q.norm": 1 + rnd(D, s=0.2),
                           p + "mix.temp": 1 + rnd(H, s=0.2), p + "mix.o": rnd(W, H * V, s=(H * V) ** -0.5)})
                 if m.get("kv_from") is None:
