@@ -74,12 +74,15 @@ int hm_relu_squared(int dtype, const void* z, int64_t z_stride, void* out, int64
  *   q_out [T, H, D].
  * q_head_w / k_head_w != NULL ([D], one row shared by the heads): before the rotation every q (k) head is divided by its
  * own RMS and multiplied by that row; q_head_scale != NULL (f32 [H]): query head h times q_head_scale[h] after it.
- * k_cache == v_cache == NULL: the rows hold q only (keys and values are another layer's), nothing is stored. */
+ * k_cache == v_cache == NULL: the rows hold q only (keys and values are another layer's), nothing is stored.
+ * interleaved: the rotation pairs channel 2i with 2i + 1 instead of i with i + rot_half; rot_mag multiplies every cosine
+ * and sine (1 = a pure rotation; inv_freq may hold any table, e.g. one rescaled for longer contexts); v_unit_norm: every
+ * value head is divided by sqrt(mean(head^2) + eps), no weight, before it is stored (not together with v_first). */
 int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, int H, int G, int D, int V, const void* q_norm_w,
                    const void* k_norm_w, float eps, const float* inv_freq, int rot_half, int unit_norm, const int32_t* tok_pos,
                    const int32_t* slot_mapping, void* k_cache, void* v_cache, const void* v_first, int64_t v_first_stride,
                    const float* lam, void* q_out, int64_t T, const void* q_head_w, const void* k_head_w,
-                   const float* q_head_scale, void* stream);
+                   const float* q_head_scale, int interleaved, float rot_mag, int v_unit_norm, void* stream);
 
 /* Attention of q [T, H, D] over the paged caches, any sizes, f32 arithmetic: the token at position i sees key j <= i,
  * and with window > 0 only if i - j < window or j < keep_first.  sink != NULL (f32 [H]): exp(sink[h]) joins the softmax
@@ -87,11 +90,15 @@ int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, int H, int G,
  * Pooled blocks (pool > 0, needs window > 0 and keep_first == 0): beside its window the token at position i sees one
  * key and value for every block of `pool` tokens whose last token lies at or before i - window: the block's mean key and
  * mean value, row e % pool_rows of page block_table[e / pool_rows] of kp_cache [pages, pool_rows, G, D] and vp_cache
- * [pages, pool_rows, G, V] for block e (pool_rows * pool >= block_size); they share the softmax with the tokens. */
+ * [pages, pool_rows, G, V] for block e (pool_rows * pool >= block_size); they share the softmax with the tokens.
+ * chunk > 0 (chunked mask; without kept first tokens and pooled blocks): the token at position i sees key j <= i only if
+ * i / chunk == j / chunk, chunks counted from position 0 of the sequence.
+ * sigmoid_w (without sink and pooled blocks): the weight of a visible key is sigmoid(score * scale + head_bias[h])
+ * (head_bias f32 [H], NULL = 0) and the weights are not normalised over the keys. */
 int hm_attn_rows(int dtype, const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                  const int32_t* tok_seq, const int32_t* tok_pos, const float* sink, int window, int keep_first, float scale,
                  void* o, int64_t T, int H, int G, int D, int V, int block_size, int max_blocks, const void* kp_cache,
-                 const void* vp_cache, int pool, int pool_rows, void* stream);
+                 const void* vp_cache, int pool, int pool_rows, int chunk, const float* head_bias, int sigmoid_w, void* stream);
 
 /* The mean key and mean value of every block of `pool` tokens that the step completes, as the caches hold them (f32
  * sums), written to the pooled caches (layout above).  Sequence b's portion covers positions [seq_pos0[b], ctx_lens[b]);
@@ -105,7 +112,7 @@ int hm_pool_blocks(int dtype, const void* k_cache, const void* v_cache, void* kp
 int hm_attn_tiles(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables, const int32_t* qstart,
                   const int32_t* seq_pos0, const float* sink, int window, int keep_first, float scale, void* o, int B, int max_q,
                   int H, int G, int D, int V, int block_size, int max_blocks, const void* kp_cache, const void* vp_cache, int pool,
-                  int pool_rows, void* stream);
+                  int pool_rows, int chunk, const float* head_bias, int sigmoid_w, void* stream);
 /* Single-token queries (q [B, H, D], ctx[b] = keys of sequence b incl. the new one): the visible key tiles are split
  * over `splits` workgroups per (sequence, key/value head) and merged in split order by a second launch.  At most 32
  * query heads per key/value head.  workspace: hm_attn_decode_workspace_bytes(B, H, V, splits) bytes. */
@@ -113,7 +120,7 @@ size_t hm_attn_decode_workspace_bytes(int64_t B, int H, int V, int splits);
 int hm_attn_decode(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables, const int32_t* ctx,
                    const float* sink, int window, int keep_first, float scale, void* o, int64_t B, int H, int G, int D, int V,
                    int block_size, int max_blocks, int splits, void* workspace, size_t workspace_bytes, const void* kp_cache,
-                   const void* vp_cache, int pool, int pool_rows, void* stream);
+                   const void* vp_cache, int pool, int pool_rows, int chunk, const float* head_bias, int sigmoid_w, void* stream);
 
 /* prep [T, H, 5, D] f32 = decay | a*u | u | k | r from the columns r_off, k_off, a_off (H*D wide) and z_off (rank wide) of
  * proj:  decay = exp(-decay_scale * sigmoid(w2 tanh(z) + w0)), a = sigmoid(a_pre + a_bias), u = k / sqrt(sum k^2 + unit_eps)
@@ -133,6 +140,25 @@ int hm_delta_recurrence(int dtype, const float* prep, const void* v, int64_t v_s
 /* out[t, h*D + i] = o[t, h, i] / sqrt(mean_i o[t, h]^2 + eps) * norm_w[h*D + i] * sigmoid(g[t, h*D + i]). */
 int hm_delta_gate_norm(int dtype, const float* o, const void* g, int64_t g_stride, const void* norm_w, float eps, void* out,
                        int64_t T, int H, int D, void* stream);
+
+/* Linear attention with a constant decay per head.  q, k [T, H*D] and v [T, H*V] are the columns q_off, k_off, v_off of
+ * proj (rows row_stride apart) passed through silu.  For every sequence b and head, over the tokens of its portion:
+ *   S <- decay[h] S + k v^T;  o[t] = S^T q
+ * state f32 [slots, H, D, V] is read at the start unless seq_pos0[b] == 0 (then S = 0) and written at the end.  decay f32
+ * [H].  o f32 [T, H, V].  D <= 256.  max_q = the longest portion of the step (a hint for staging only). */
+int hm_lightning_recurrence(int dtype, const void* proj, int64_t row_stride, int q_off, int k_off, int v_off,
+                            const float* decay, float* state, const int32_t* qstart, const int32_t* seq_pos0,
+                            const int32_t* seq_slot, float* o, int B, int H, int D, int V, int max_q, void* stream);
+
+/* The boundary between two sublayers of a residual whose sublayers sit between two Dynamic-Tanh norms,
+ * dyt(z) = tanh(alpha[0] z) * w + b per channel (alpha f32 on the device, w and b in the storage type); x [T, W] f32 is
+ * updated in place, one elementwise launch:
+ *   y != NULL, ids == NULL:  x[t] += dyt_post(y[t])
+ *   y != NULL, ids != NULL:  x[t]  = y[ids[t]]                             (y = an embedding table; no norm)
+ *   h_out != NULL:           h_out[t] = next_w ? dyt_next(x[t]) : x[t], in the storage type. */
+int hm_dyt_residual(int dtype, float* x, const void* y, const int64_t* ids, const void* post_w, const void* post_b,
+                    const float* post_alpha, const void* next_w, const void* next_b, const float* next_alpha, void* h_out,
+                    int64_t T, int W, void* stream);
 
 /* The boundary between two sublayers of a residual that is normalised on the sublayers' OUTPUT, with an RMS norm over
  * `groups` equal consecutive parts of the vector (each part divided by its own sqrt(mean(part^2) + eps)); x [T, W] f32 is

@@ -31,6 +31,7 @@ extern "C" {
 #define SM_ACT_CLAMPED_GLU 0
 #define SM_ACT_GELU 1
 #define SM_ACT_GELU_TANH 2
+#define SM_ACT_SILU_GLU 3
 
 #define SM_OK 0
 #define SM_EINVAL (-1)
@@ -65,6 +66,10 @@ int sm_canon_conv(int dtype, const void* h, const void* w, const void* state, in
 /* state[slot, run] <- the last taps-1 inputs of every sequence after this step (older ones shift out). */
 int sm_canon_update(int dtype, const void* h, void* state, int run, int runs, const int32_t* qstart,
                     const int32_t* seq_slot, int B, int W, int taps, void* stream);
+
+/* out[t] = x[t] / sqrt(mean(x[t]^2) + eps) * w over R columns, x rows row_stride apart, out dense [T, R]. */
+int sm_rms_norm_rows(int dtype, const void* x, int64_t row_stride, const void* w, float eps, void* out, int64_t T, int R,
+                     void* stream);
 
 /* c = x / sqrt(mean(x^2) + eps) * w over R columns of rows with stride `row_stride` elements; stored at cache row
  * slot_mapping[t] of a paged cache [rows, R] (slot < 0: skipped). */
@@ -119,15 +124,18 @@ int sm_clamped_glu(int dtype, const void* gu, float limit, float alpha, void* ou
  * eligible experts with the largest s are chosen, weights = their s / (sum + 1e-20).  idx [T, top] i32, wts [T, top] f32. */
 /* score = SM_ROUTE_SIGMOID: s = sigmoid(z) instead.  correction != NULL (f32 [E]): the choice (groups and experts) goes
  * by s + correction, the weights stay s.  group_top (1..4): a group scores the sum of its group_top largest choice
- * scores.  renorm == 0: the weights are the chosen s as they are. */
+ * scores.  renorm == 0: the weights are the chosen s as they are.  bias != NULL (f32 [E]): z = router_w h + bias (with
+ * softmax scores and renorm the weights are then the softmax over the chosen experts' logits). */
 int sm_moe_route(int dtype, const void* h, const float* router_w, int32_t* idx, float* wts, int64_t T, int W, int E,
-                 int top, int groups, int keep, int score, const float* correction, int group_top, int renorm, void* stream);
+                 int top, int groups, int keep, int score, const float* correction, int group_top, int renorm,
+                 const float* bias, void* stream);
 
 /* Expert products, one (token, chosen expert) pair at a time (memory-bound form for few tokens):
  * act[p] = clamped_glu(w_gu[e] h[t]) with w_gu [E, 2F, W] (gate rows, then up rows), p = t * top + k; then
  * y[t] = sum_k wts[t, k] * (w_down[e_k] act[t * top + k]) + shared[t]   (w_down [E, W, F]; shared may be NULL). */
 /* act_kind = SM_ACT_CLAMPED_GLU as above; SM_ACT_GELU / SM_ACT_GELU_TANH: an expert is w_down act(w_up h) with the exact
- * (erf) or the tanh GELU, and w_gu is [E, F, W] (one part when tiled). */
+ * (erf) or the tanh GELU, and w_gu is [E, F, W] (one part when tiled).  SM_ACT_SILU_GLU: the gated form without the one,
+ * g' sigmoid(alpha g') u' (limit = +inf, alpha = 1: silu(gate) * up), w_gu as for the clamped GLU. */
 int sm_moe_pairs_gate_up(int dtype, const void* h, const int32_t* idx, const void* w_gu, float limit, float alpha,
                          int act_kind, void* act, int64_t T, int top, int W, int F, void* stream);
 int sm_moe_pairs_down(int dtype, const void* act, const int32_t* idx, const float* wts, const void* w_down,

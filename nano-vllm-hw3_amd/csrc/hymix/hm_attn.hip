@@ -17,7 +17,8 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ 
                                                           const int32_t* __restrict__ slot_mapping, T* __restrict__ k_cache,
                                                           T* __restrict__ v_cache, const T* __restrict__ v_first,
                                                           int64_t v_first_stride, const float* __restrict__ lam,
-                                                          T* __restrict__ q_out) {
+                                                          T* __restrict__ q_out, int interleaved, float rot_mag,
+                                                          int v_unit_norm) {
     extern __shared__ float qk[];
     __shared__ float red[16];
     const int64_t t = blockIdx.x;
@@ -66,15 +67,22 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ 
     // the angles depend on the channel pair alone: one sine and cosine per pair, shared by all heads
     float* cs = qk + nq + nk;
     const float pos = (float)tok_pos[t];
-    for (int i = tid; i < rot_half; i += 256) sincosf(pos * inv_freq[i], cs + rot_half + i, cs + i);
+    for (int i = tid; i < rot_half; i += 256) {
+        float sn, cn;
+        sincosf(pos * inv_freq[i], &sn, &cn);
+        cs[i] = cn * rot_mag;                  // (rot_mag = 1 leaves them as they are)
+        cs[rot_half + i] = sn * rot_mag;
+    }
     __syncthreads();
     for (int e = tid; e < (H + G) * rot_half; e += 256) {       // one thread per rotated pair
         const int hh = e / rot_half, i = e - hh * rot_half;
         const float c = cs[i], s = cs[rot_half + i];
         float* p = qk + (size_t)hh * D;
-        const float a = p[i], b = p[i + rot_half];
-        p[i] = a * c - b * s;
-        p[i + rot_half] = b * c + a * s;
+        // channel i pairs with channel i + rot_half, or (interleaved) channel 2i with channel 2i + 1
+        const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + rot_half;
+        const float a = p[ia], b = p[ib];
+        p[ia] = a * c - b * s;
+        p[ib] = b * c + a * s;
     }
     __syncthreads();
     if (unit_norm) {                           // every head divided by its RMS; one wave per head
@@ -103,7 +111,17 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(const T* __restrict__ 
         *(Pack*)(k_cache + (size_t)slot * nk + c) = pk;
     }
     const T* vr = row + nq + nk;
-    if (v_first != nullptr) {
+    if (v_unit_norm) {                         // every value head divided by its RMS (no weight); one wave per head
+        for (int gg = wave; gg < G; gg += 4) {
+            const T* p = vr + (size_t)gg * V;
+            float ss = 0.f;
+            for (int i = lane; i < V; i += 64) { const float v = to_f(p[i]); ss += v * v; }
+            ss = wave_sum(ss);
+            const float r = 1.f / sqrtf(ss / (float)V + eps);
+            T* dst = v_cache + (size_t)slot * nv + (size_t)gg * V;
+            for (int i = lane; i < V; i += 64) dst[i] = from_f<T>(to_f(p[i]) * r);
+        }
+    } else if (v_first != nullptr) {
         const float l = lam[0];
         const T* fr = v_first + (size_t)t * v_first_stride;
         for (int c = tid * VEC; c < nv; c += 256 * VEC) {
@@ -130,14 +148,16 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const T* __restrict__ q,
                                                         const float* __restrict__ sink, int window, int keep_first, float scale,
                                                         T* __restrict__ o, int H, int G, int D, int V, int block_size,
                                                         int max_blocks, const T* __restrict__ kp_cache,
-                                                        const T* __restrict__ vp_cache, int pool, int pool_rows) {
+                                                        const T* __restrict__ vp_cache, int pool, int pool_rows, int chunk,
+                                                        const float* __restrict__ head_bias, int sigmoid_w) {
     extern __shared__ float q_lds[];                 // D floats
     __shared__ float s_lds[kRowChunk];
     __shared__ int row_lds[kRowChunk];
     const int64_t t = blockIdx.x;
     const int hd = blockIdx.y, g = hd / (H / G);
     const int b = tok_seq[t], n = tok_pos[t] + 1;    // keys 0 .. n-1 are causal
-    const int lo = window > 0 ? max(0, n - window) : 0;
+    // the first visible key: the window's start, or (chunked mask) the start of the query's own chunk of positions
+    const int lo = max(window > 0 ? max(0, n - window) : 0, chunk > 0 ? (n - 1) / chunk * chunk : 0);
     const int kept = window > 0 ? min(keep_first, lo) : 0;
     const int seen = pooled_seen(n - 1, window, pool);       // pooled blocks that lie wholly before the window
     const int total = seen + kept + (n - lo);
@@ -171,6 +191,20 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const T* __restrict__ q,
             if (lane == 0) s_lds[kk] = row != -1 ? d * scale : -INFINITY;
         }
         __syncthreads();
+        if (sigmoid_w) {                             // independent weights sigmoid(score + bias), not normalised over keys
+            const float hb = head_bias ? head_bias[hd] : 0.f;
+            for (int kk = 0; kk < kRowChunk; ++kk) {
+                const int row = row_lds[kk];
+                if (row == -1) break;
+                const float p = sigmoid_f(s_lds[kk] + hb);
+                const T* vr = v_cache + ((size_t)row * G + g) * V;
+                for (int r = 0; r < 4; ++r) {
+                    const int c = tid + 256 * r;
+                    if (c < V) acc[r] += p * to_f(vr[c]);
+                }
+            }
+            continue;
+        }
         float mx = m_run;
         for (int kk = 0; kk < kRowChunk; ++kk) mx = fmaxf(mx, s_lds[kk]);
         const float alpha = expf(m_run - mx);        // first chunk: exp(-inf) = 0
@@ -191,7 +225,9 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(const T* __restrict__ q,
         m_run = mx;
     }
     float inv;
-    if (sink != nullptr) {                           // one more term in the denominator, no value
+    if (sigmoid_w) {
+        inv = 1.f;
+    } else if (sink != nullptr) {                    // one more term in the denominator, no value
         const float sk = sink[hd], mx = fmaxf(m_run, sk), alpha = expf(m_run - mx);
         for (int r = 0; r < 4; ++r) acc[r] *= alpha;
         inv = 1.f / (l_run * alpha + expf(sk - mx));
@@ -276,12 +312,13 @@ extern "C" int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, in
                               const void* k_norm_w, float eps, const float* inv_freq, int rot_half, int unit_norm,
                               const int32_t* tok_pos, const int32_t* slot_mapping, void* k_cache, void* v_cache,
                               const void* v_first, int64_t v_first_stride, const float* lam, void* q_out, int64_t T,
-                              const void* q_head_w, const void* k_head_w, const float* q_head_scale, void* stream) {
+                              const void* q_head_w, const void* k_head_w, const float* q_head_scale, int interleaved,
+                              float rot_mag, int v_unit_norm, void* stream) {
     const bool q_only = !k_cache && !v_cache;
     if (T < 0 || H < 1 || G < 1 || D < 1 || V < 1 || H % G != 0 || rot_half < 0 || 2 * rot_half > D ||
         row_stride < (q_only ? (int64_t)H * D : (int64_t)(H + G) * D + (int64_t)G * V) || (!q_norm_w) != (!k_norm_w) ||
         (rot_half > 0 && !inv_freq) || (v_first && (!lam || v_first_stride < (int64_t)G * V)) || (!k_cache) != (!v_cache) ||
-        (q_only && (v_first || k_norm_w)) || (q_head_w && !q_only && !k_head_w) ||
+        (q_only && (v_first || k_norm_w)) || (q_head_w && !q_only && !k_head_w) || (v_unit_norm && v_first) ||
         (T > 0 && (!qkv || !tok_pos || !slot_mapping || !q_out))) {
         set_error("hm_qkv_prepare: bad argument");
         return HM_EINVAL;
@@ -298,7 +335,8 @@ extern "C" int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, in
     hipLaunchKernelGGL((qkv_prepare_kernel<DT, VEC_>), dim3((unsigned)T), dim3(256), lds, as_stream(stream), (const DT*)qkv,  \
                        row_stride, H, G, D, V, (const DT*)q_norm_w, (const DT*)k_norm_w, (const DT*)q_head_w,                 \
                        (const DT*)k_head_w, q_head_scale, eps, inv_freq, rot_half, unit_norm,                                 \
-                       tok_pos, slot_mapping, (DT*)k_cache, (DT*)v_cache, (const DT*)v_first, v_first_stride, lam, (DT*)q_out)
+                       tok_pos, slot_mapping, (DT*)k_cache, (DT*)v_cache, (const DT*)v_first, v_first_stride, lam, (DT*)q_out, \
+                       interleaved, rot_mag, v_unit_norm)
     HM_DISPATCH(dtype, "hm_qkv_prepare", if (wide && bits % (8 * sizeof(DT)) == 0) HM_PREP(8); else HM_PREP(1));
 #undef HM_PREP
     HM_CHECK_LAUNCH("hm_qkv_prepare");
@@ -308,8 +346,10 @@ extern "C" int hm_qkv_prepare(int dtype, const void* qkv, int64_t row_stride, in
 extern "C" int hm_attn_rows(int dtype, const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                             const int32_t* tok_seq, const int32_t* tok_pos, const float* sink, int window, int keep_first,
                             float scale, void* o, int64_t T, int H, int G, int D, int V, int block_size, int max_blocks,
-                            const void* kp_cache, const void* vp_cache, int pool, int pool_rows, void* stream) {
+                            const void* kp_cache, const void* vp_cache, int pool, int pool_rows, int chunk, const float* head_bias,
+                            int sigmoid_w, void* stream) {
     if (T < 0 || H < 1 || G < 1 || H % G != 0 || D < 1 || V < 1 || block_size < 1 || max_blocks < 1 || window < 0 || keep_first < 0 ||
+        chunk < 0 || (chunk > 0 && (keep_first > 0 || pool > 0)) || (sigmoid_w && (sink || pool > 0)) || (head_bias && !sigmoid_w) ||
         pool < 0 || (pool > 0 && (!kp_cache || !vp_cache || window < 1 || keep_first > 0 || pool_rows * pool < block_size)) ||
         (T > 0 && (!q || !k_cache || !v_cache || !block_tables || !tok_seq || !tok_pos || !o))) {
         set_error("hm_attn_rows: bad argument");
@@ -322,7 +362,7 @@ extern "C" int hm_attn_rows(int dtype, const void* q, const void* k_cache, const
                 hipLaunchKernelGGL(attn_rows_kernel<DT>, grid, dim3(256), (size_t)D * 4, as_stream(stream), (const DT*)q,
                                    (const DT*)k_cache, (const DT*)v_cache, block_tables, tok_seq, tok_pos, sink, window,
                                    keep_first, scale, (DT*)o, H, G, D, V, block_size, max_blocks, (const DT*)kp_cache,
-                                   (const DT*)vp_cache, pool, pool_rows));
+                                   (const DT*)vp_cache, pool, pool_rows, chunk, head_bias, sigmoid_w));
     HM_CHECK_LAUNCH("hm_attn_rows");
     return HM_OK;
 }

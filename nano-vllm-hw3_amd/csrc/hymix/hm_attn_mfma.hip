@@ -8,7 +8,7 @@
 
 namespace hm {
 
-template <int NBK, int NBV>
+template <int NBK, int NBV, bool SIG>
 __global__ __launch_bounds__(256) void attn_tiles_kernel(const unsigned short* __restrict__ q, const unsigned short* __restrict__ kc,
                                                          const unsigned short* __restrict__ vc,
                                                          const int32_t* __restrict__ block_tables,
@@ -16,7 +16,8 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const unsigned short* _
                                                          const float* __restrict__ sink, int window, int keep_first, float scale,
                                                          unsigned short* __restrict__ o, int H, int G, int D, int V, int block_size,
                                                          int max_blocks, const unsigned short* __restrict__ kp,
-                                                         const unsigned short* __restrict__ vp, int pool, int pool_rows) {
+                                                         const unsigned short* __restrict__ vp, int pool, int pool_rows,
+                                                         int chunk, const float* __restrict__ head_bias) {
     __shared__ __attribute__((aligned(16))) unsigned char lds_k[TileGeom<NBK>::LDS_BYTES];
     __shared__ __attribute__((aligned(16))) unsigned char lds_v[TileGeom<NBV>::LDS_BYTES];
     const int b = blockIdx.y, g = blockIdx.z, rep = H / G;
@@ -32,17 +33,19 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const unsigned short* _
     const int row_pos = pos0 + tok;
     const int wave_min_pos = pos0 + min(tile0 + 32 * wave, rows - 1) / rep;
     const int n_keys = pos0 + min(tile0 + 127, rows - 1) / rep + 1;
-    const TileWalk walk = make_walk(pos0 + tile0 / rep, n_keys - 1, window, keep_first, pool);
+    const TileWalk walk = make_walk(pos0 + tile0 / rep, n_keys - 1, window, keep_first, pool, chunk);
     const float c_log2 = scale * 1.4426950408889634f;
+    const float bias_log2 = (SIG && head_bias) ? head_bias[head] * 1.4426950408889634f : 0.f;
     f32x16 oacc[NBV];
     float m_run, l_tot;
-    kv_tile_loop<NBK, NBV, 4>(q + ((size_t)(q0 + tok) * H + head) * D, kc, vc, block_tables + (size_t)b * max_blocks, D, V, G, g,
-                              block_size, walk, 0, walk.count(n_keys), n_keys, row_pos, wave_min_pos, window, keep_first, c_log2,
-                              kp, vp, pool, pool_rows, lds_k, lds_v, oacc, m_run, l_tot);
+    kv_tile_loop<NBK, NBV, 4, SIG>(q + ((size_t)(q0 + tok) * H + head) * D, kc, vc, block_tables + (size_t)b * max_blocks, D, V, G, g,
+                                   block_size, walk, 0, walk.count(n_keys), n_keys, row_pos, wave_min_pos, window, keep_first, c_log2,
+                                   kp, vp, pool, pool_rows, lds_k, lds_v, oacc, m_run, l_tot, chunk, bias_log2);
     if (r >= rows) return;
-    // the sink joins the denominator with its own score, which is not scaled (m_run is finite: a row sees itself)
+    // the sink joins the denominator with its own score, which is not scaled (m_run is finite: a row sees itself);
+    // sigmoid weights are not normalised
     const float den = l_tot + (sink ? expf(sink[head] - m_run * scale) : 0.f);
-    const float inv = 1.f / den;
+    const float inv = SIG ? 1.f : 1.f / den;
     unsigned short* op = o + ((size_t)(q0 + tok) * H + head) * V + 4 * hi;
 #pragma unroll
     for (int d = 0; d < NBV; ++d)
@@ -59,19 +62,20 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(const unsigned short* _
 // floats per (sequence, split, head) in the workspace: maximum in log2 units, sum, then the padded outputs
 __host__ __device__ constexpr int part_stride(int nbv) { return 32 * nbv + 2; }
 
-template <int NBK, int NBV>
+template <int NBK, int NBV, bool SIG>
 __global__ __launch_bounds__(64) void attn_decode_kernel(const unsigned short* __restrict__ q, const unsigned short* __restrict__ kc,
                                                          const unsigned short* __restrict__ vc,
                                                          const int32_t* __restrict__ block_tables, const int32_t* __restrict__ ctx,
                                                          int window, int keep_first, float scale, float* __restrict__ ws, int H,
                                                          int G, int D, int V, int block_size, int max_blocks, int splits,
                                                          const unsigned short* __restrict__ kp,
-                                                         const unsigned short* __restrict__ vp, int pool, int pool_rows) {
+                                                         const unsigned short* __restrict__ vp, int pool, int pool_rows, int chunk,
+                                                         const float* __restrict__ head_bias) {
     __shared__ __attribute__((aligned(16))) unsigned char lds_k[TileGeom<NBK>::LDS_BYTES];
     __shared__ __attribute__((aligned(16))) unsigned char lds_v[TileGeom<NBV>::LDS_BYTES];
     const int sp = blockIdx.x, b = blockIdx.y, g = blockIdx.z, rep = H / G;
     const int n = ctx[b];
-    const TileWalk walk = make_walk(n - 1, n - 1, window, keep_first, pool);
+    const TileWalk walk = make_walk(n - 1, n - 1, window, keep_first, pool, chunk);
     const int nt = walk.count(n), per = (nt + splits - 1) / splits;
     const int vt_lo = sp * per, vt_hi = min(nt, vt_lo + per);
     const int lane = threadIdx.x & 63, l31 = lane & 31, hi = lane >> 5;
@@ -84,9 +88,10 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(const unsigned short* _
     const float c_log2 = scale * 1.4426950408889634f;
     f32x16 oacc[NBV];
     float m_run, l_tot;
-    kv_tile_loop<NBK, NBV, 1>(q + ((size_t)b * H + head) * D, kc, vc, block_tables + (size_t)b * max_blocks, D, V, G, g, block_size,
-                              walk, vt_lo, vt_hi, n, n - 1, n - 1, window, keep_first, c_log2, kp, vp, pool, pool_rows, lds_k, lds_v,
-                              oacc, m_run, l_tot);
+    const float bias_log2 = (SIG && head_bias) ? head_bias[head] * 1.4426950408889634f : 0.f;
+    kv_tile_loop<NBK, NBV, 1, SIG>(q + ((size_t)b * H + head) * D, kc, vc, block_tables + (size_t)b * max_blocks, D, V, G, g,
+                                   block_size, walk, vt_lo, vt_hi, n, n - 1, n - 1, window, keep_first, c_log2, kp, vp, pool,
+                                   pool_rows, lds_k, lds_v, oacc, m_run, l_tot, chunk, bias_log2);
     if (l31 >= rep) return;
     if (hi == 0) { part[0] = l_tot > 0.f ? m_run * c_log2 : -INFINITY; part[1] = l_tot; }
 #pragma unroll
@@ -98,9 +103,20 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(const unsigned short* _
 }
 
 __global__ void attn_decode_merge_kernel(const float* __restrict__ ws, const float* __restrict__ sink,
-                                         unsigned short* __restrict__ o, int H, int V, int splits, int stride) {
+                                         unsigned short* __restrict__ o, int H, int V, int splits, int stride, int plain_sum) {
     const size_t row = blockIdx.x;                          // b * H + h
     const size_t b = row / H, h = row % H;
+    if (plain_sum) {                                        // weights that are not normalised: the splits' outputs add up
+        for (int c = threadIdx.x; c < V; c += blockDim.x) {
+            float acc = 0.f;
+            for (int s = 0; s < splits; ++s) {
+                const float* p = ws + ((b * splits + s) * H + h) * stride;
+                if (p[1] > 0.f) acc += p[2 + c];
+            }
+            o[row * V + c] = __builtin_bit_cast(unsigned short, (bf16_t)acc);
+        }
+        return;
+    }
     const float sk = sink ? sink[h] * 1.4426950408889634f : -INFINITY;       // in log2 units, as the partial maxima
     float M = sk;
     for (int s = 0; s < splits; ++s) {
@@ -141,18 +157,26 @@ static bool shape_ok(int H, int G, int D, int V, int block_size) {
 
 using namespace hm;
 
-// run `stmt` with NBK_ / NBV_ bound to the padded head sizes
-#define HM_BY_HEAD_SIZE(nbk, nbv, M)                                              \
+// run M with K_ / V_ bound to the padded head sizes ...
+#define HM_BY_HEAD_SIZE_(nbk, nbv, M, S)                                          \
     do {                                                                          \
-        if (nbk == 1) { if (nbv == 1) M(1, 1); else if (nbv == 2) M(1, 2); else M(1, 4); } \
-        else if (nbk == 2) { if (nbv == 1) M(2, 1); else if (nbv == 2) M(2, 2); else M(2, 4); } \
-        else { if (nbv == 1) M(4, 1); else if (nbv == 2) M(4, 2); else M(4, 4); } \
+        if (nbk == 1) { if (nbv == 1) M(1, 1, S); else if (nbv == 2) M(1, 2, S); else M(1, 4, S); } \
+        else if (nbk == 2) { if (nbv == 1) M(2, 1, S); else if (nbv == 2) M(2, 2, S); else M(2, 4, S); } \
+        else { if (nbv == 1) M(4, 1, S); else if (nbv == 2) M(4, 2, S); else M(4, 4, S); } \
     } while (0)
+// ... and S_ to the kind of weights (softmax or sigmoid)
+#define HM_BY_HEAD_SIZE(nbk, nbv, sig, M)                                         \
+    do { if (sig) HM_BY_HEAD_SIZE_(nbk, nbv, M, true); else HM_BY_HEAD_SIZE_(nbk, nbv, M, false); } while (0)
 
 extern "C" int hm_attn_tiles(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_tables,
                              const int32_t* qstart, const int32_t* seq_pos0, const float* sink, int window, int keep_first,
                              float scale, void* o, int B, int max_q, int H, int G, int D, int V, int block_size, int max_blocks,
-                             const void* kp_cache, const void* vp_cache, int pool, int pool_rows, void* stream) {
+                             const void* kp_cache, const void* vp_cache, int pool, int pool_rows, int chunk,
+                             const float* head_bias, int sigmoid_w, void* stream) {
+    if (chunk < 0 || (chunk > 0 && (keep_first > 0 || pool > 0)) || (sigmoid_w && (sink || pool > 0)) || (head_bias && !sigmoid_w)) {
+        set_error("hm_attn_tiles: a chunked mask goes without kept first tokens and pooled blocks, sigmoid weights without sink and pooled blocks");
+        return HM_EINVAL;
+    }
     if (B < 0 || max_q < 0 || H < 1 || G < 1 || D < 1 || V < 1 || block_size < 1 || max_blocks < 1 || window < 0 || keep_first < 0 ||
         !pool_args_ok(kp_cache, vp_cache, pool, pool_rows, window, keep_first, block_size) ||
         (B > 0 && max_q > 0 && (!q || !k_cache || !v_cache || !block_tables || !qstart || !seq_pos0 || !o))) {
@@ -168,12 +192,12 @@ extern "C" int hm_attn_tiles(const void* q, const void* k_cache, const void* v_c
     dim3 grid((unsigned)tiles, (unsigned)B, (unsigned)G), block(256);
     hipStream_t s = as_stream(stream);
     const int nbk = padded_nb(D), nbv = padded_nb(V);
-#define HM_TILES(K_, V_)                                                                                                     \
-    hipLaunchKernelGGL((attn_tiles_kernel<K_, V_>), grid, block, 0, s, (const unsigned short*)q, (const unsigned short*)k_cache, \
+#define HM_TILES(K_, V_, S_)                                                                                                 \
+    hipLaunchKernelGGL((attn_tiles_kernel<K_, V_, S_>), grid, block, 0, s, (const unsigned short*)q, (const unsigned short*)k_cache, \
                        (const unsigned short*)v_cache, block_tables, qstart, seq_pos0, sink, window, keep_first, scale,       \
                        (unsigned short*)o, H, G, D, V, block_size, max_blocks, (const unsigned short*)kp_cache,               \
-                       (const unsigned short*)vp_cache, pool, pool_rows)
-    HM_BY_HEAD_SIZE(nbk, nbv, HM_TILES);
+                       (const unsigned short*)vp_cache, pool, pool_rows, chunk, head_bias)
+    HM_BY_HEAD_SIZE(nbk, nbv, sigmoid_w, HM_TILES);
 #undef HM_TILES
     HM_CHECK_LAUNCH("hm_attn_tiles");
     return HM_OK;
@@ -188,7 +212,11 @@ extern "C" int hm_attn_decode(const void* q, const void* k_cache, const void* v_
                               const int32_t* ctx, const float* sink, int window, int keep_first, float scale, void* o, int64_t B,
                               int H, int G, int D, int V, int block_size, int max_blocks, int splits, void* workspace,
                               size_t workspace_bytes, const void* kp_cache, const void* vp_cache, int pool, int pool_rows,
-                              void* stream) {
+                              int chunk, const float* head_bias, int sigmoid_w, void* stream) {
+    if (chunk < 0 || (chunk > 0 && (keep_first > 0 || pool > 0)) || (sigmoid_w && (sink || pool > 0)) || (head_bias && !sigmoid_w)) {
+        set_error("hm_attn_decode: a chunked mask goes without kept first tokens and pooled blocks, sigmoid weights without sink and pooled blocks");
+        return HM_EINVAL;
+    }
     if (B < 0 || H < 1 || G < 1 || D < 1 || V < 1 || block_size < 1 || max_blocks < 1 || splits < 1 || window < 0 || keep_first < 0 ||
         !pool_args_ok(kp_cache, vp_cache, pool, pool_rows, window, keep_first, block_size) ||
         (B > 0 && (!q || !k_cache || !v_cache || !block_tables || !ctx || !o || !workspace))) {
@@ -207,16 +235,16 @@ extern "C" int hm_attn_decode(const void* q, const void* k_cache, const void* v_
     dim3 grid((unsigned)splits, (unsigned)B, (unsigned)G);
     hipStream_t s = as_stream(stream);
     const int nbk = padded_nb(D), nbv = padded_nb(V);
-#define HM_DEC(K_, V_)                                                                                                        \
-    hipLaunchKernelGGL((attn_decode_kernel<K_, V_>), grid, dim3(64), 0, s, (const unsigned short*)q, (const unsigned short*)k_cache, \
+#define HM_DEC(K_, V_, S_)                                                                                                    \
+    hipLaunchKernelGGL((attn_decode_kernel<K_, V_, S_>), grid, dim3(64), 0, s, (const unsigned short*)q, (const unsigned short*)k_cache, \
                        (const unsigned short*)v_cache, block_tables, ctx, window, keep_first, scale, (float*)workspace, H, G, D, \
                        V, block_size, max_blocks, splits, (const unsigned short*)kp_cache, (const unsigned short*)vp_cache, pool, \
-                       pool_rows)
-    HM_BY_HEAD_SIZE(nbk, nbv, HM_DEC);
+                       pool_rows, chunk, head_bias)
+    HM_BY_HEAD_SIZE(nbk, nbv, sigmoid_w, HM_DEC);
 #undef HM_DEC
     HM_CHECK_LAUNCH("hm_attn_decode");
     hipLaunchKernelGGL(attn_decode_merge_kernel, dim3((unsigned)(B * H)), dim3(64), 0, s, (const float*)workspace, sink,
-                       (unsigned short*)o, H, V, splits, part_stride(nbv));
+                       (unsigned short*)o, H, V, splits, part_stride(nbv), sigmoid_w);
     HM_CHECK_LAUNCH("hm_attn_decode (merge)");
     return HM_OK;
 }

@@ -47,13 +47,15 @@ struct TileWalk {
 };
 
 // min_pos / max_pos = the smallest / largest position among the rows that walk together
-__device__ __forceinline__ TileWalk make_walk(int min_pos, int max_pos, int window, int keep_first, int pool) {
+// chunk > 0: a row also sees nothing before the start of its own chunk of `chunk` positions
+__device__ __forceinline__ TileWalk make_walk(int min_pos, int max_pos, int window, int keep_first, int pool, int chunk = 0) {
     TileWalk w;
     w.n_pool = pooled_seen(max_pos, window, pool);
     w.pool_tiles = (w.n_pool + kTileKeys - 1) / kTileKeys;
-    if (window <= 0) { w.keep_tiles = 0; w.win_lo = 0; return w; }
-    w.win_lo = max(0, min_pos - window + 1) / kTileKeys * kTileKeys;
-    w.keep_tiles = min((keep_first + kTileKeys - 1) / kTileKeys, w.win_lo / kTileKeys);
+    int lo = window > 0 ? max(0, min_pos - window + 1) : 0;
+    if (chunk > 0) lo = max(lo, min_pos / chunk * chunk);
+    w.win_lo = lo / kTileKeys * kTileKeys;
+    w.keep_tiles = window > 0 ? min((keep_first + kTileKeys - 1) / kTileKeys, w.win_lo / kTileKeys) : 0;
     return w;
 }
 
@@ -61,14 +63,16 @@ __device__ __forceinline__ TileWalk make_walk(int min_pos, int max_pos, int wind
 // position of the wave's rows.  Every wave of the workgroup must call this with the same tiles.  On return oacc holds the
 // unnormalised output (lane: query l & 31, columns 32 d + 8 (r >> 2) + 4 (l >> 5) + (r & 3)), m_run the row maximum of
 // the raw scores (-inf if the row saw no key) and l_tot the sum of exp2((s - m_run) * c_log2) over the row.
-template <int NBK, int NBV, int WAVES>
+// SIG: the weight of a visible key is sigmoid(score * scale + bias), bias_log2 = the row's bias times log2(e); the weights
+// are not normalised, oacc is the output itself, m_run = 0 and l_tot = 1.
+template <int NBK, int NBV, int WAVES, bool SIG = false>
 __device__ __forceinline__ void kv_tile_loop(const unsigned short* __restrict__ qrow, const unsigned short* __restrict__ kc,
                                              const unsigned short* __restrict__ vc, const int32_t* __restrict__ table, int D, int V,
                                              int G, int g, int block_size, TileWalk walk, int vt_lo, int vt_hi, int n_keys,
                                              int row_pos, int wave_min_pos, int window, int keep_first, float c_log2,
                                              const unsigned short* __restrict__ kp, const unsigned short* __restrict__ vp,
                                              int pool, int pool_rows, unsigned char* lds_k, unsigned char* lds_v, f32x16 (&oacc)[NBV], float& m_run,
-                                             float& l_tot) {
+                                             float& l_tot, int chunk = 0, float bias_log2 = 0.f) {
     typedef TileGeom<NBK> GK;
     typedef TileGeom<NBV> GV;
     constexpr int NLK = GK::CH / WAVES, NLV = GV::CH / WAVES;      // 16-byte chunks a thread stages per tile
@@ -151,6 +155,7 @@ __device__ __forceinline__ void kv_tile_loop(const unsigned short* __restrict__ 
     const int gq = (lane >> 4) & 1, ti = lane & 15, tq = ti >> 2, tp = ti & 3;      // transposed-read address pieces
 
     const int my_pool = pooled_seen(row_pos, window, pool);   // pooled entries this row sees
+    const int chunk_lo = chunk > 0 ? row_pos / chunk * chunk : 0;
     load_tile(vt_lo);
     store_tile();
     __syncthreads();
@@ -173,6 +178,12 @@ __device__ __forceinline__ void kv_tile_loop(const unsigned short* __restrict__ 
                 s[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[j], 0, 0, 0);
             }
         }
+        if (SIG) {                                           // the logit in log2 units, before the mask
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[j][r] = __builtin_fmaf(s[j][r], c_log2, bias_log2);
+        }
         if (pooled) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
@@ -181,46 +192,57 @@ __device__ __forceinline__ void kv_tile_loop(const unsigned short* __restrict__ 
                     const int e = kt0 + 32 * j + (r & 3) + 8 * (r >> 2) + 4 * hi;
                     if (e >= my_pool) s[j][r] = -INFINITY;
                 }
-        } else if (window > 0 || kt0 + kTileKeys - 1 > wave_min_pos) {
+        } else if (window > 0 || chunk > 0 || kt0 + kTileKeys - 1 > wave_min_pos) {
 #pragma unroll
             for (int j = 0; j < 2; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int key = kt0 + 32 * j + (r & 3) + 8 * (r >> 2) + 4 * hi;
-                    const bool seen = key <= row_pos && (window <= 0 || row_pos - key < window || key < keep_first);
+                    const bool seen = key <= row_pos && key >= chunk_lo &&
+                                      (window <= 0 || row_pos - key < window || key < keep_first);
                     if (!seen) s[j][r] = -INFINITY;
                 }
         }
-        float mx = s[0][0];
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[j][r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        // a row may have seen nothing yet (its window starts in a later tile): no rescale, and every weight is zero
-        const bool none = m_new == -INFINITY;
-        const float alpha = none ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new) * c_log2);
-        const float mc = none ? 0.f : m_new * c_log2;
-        float psum = 0.f;
         bf16x8 pf[2][2];
+        if (SIG) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+                for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][8 * t + e], c_log2, -mc));
-                    psum += p;
-                    pf[j][t][e] = (bf16_t)p;
-                }
-        l_run = l_run * alpha + psum;
-        m_run = m_new;
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+                    for (int e = 0; e < 8; ++e)          // a masked logit is -inf: exp2(+inf) = inf and the weight is 0
+                        pf[j][t][e] = (bf16_t)__builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-s[j][8 * t + e]));
+        } else {
+            float mx = s[0][0];
 #pragma unroll
-            for (int d = 0; d < NBV; ++d)
+            for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) oacc[d][r] *= alpha;
+                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[j][r]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run, mx);
+            // a row may have seen nothing yet (its window starts in a later tile): no rescale, and every weight is zero
+            const bool none = m_new == -INFINITY;
+            const float alpha = none ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new) * c_log2);
+            const float mc = none ? 0.f : m_new * c_log2;
+            float psum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][8 * t + e], c_log2, -mc));
+                        psum += p;
+                        pf[j][t][e] = (bf16_t)p;
+                    }
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+                for (int d = 0; d < NBV; ++d)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[d][r] *= alpha;
+            }
         }
 #pragma unroll
         for (int d = 0; d < NBV; ++d)
@@ -245,6 +267,7 @@ __device__ __forceinline__ void kv_tile_loop(const unsigned short* __restrict__ 
         }
     }
     l_tot = l_run + __shfl_xor(l_run, 32);
+    if (SIG) { m_run = 0.f; l_tot = 1.f; }
 }
 
 }  // namespace hm

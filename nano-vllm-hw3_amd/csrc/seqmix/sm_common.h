@@ -49,6 +49,14 @@ __device__ __forceinline__ float gelu_erf(float z) { return 0.5f * z * (1.f + er
 __device__ __forceinline__ float gelu_tanh(float z) {
     return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
+// the gated forms: g' = min(g, limit), u' = clamp(u, +-limit), g' sigmoid(alpha g') (u' + 1) (SM_ACT_CLAMPED_GLU), or with
+// SM_ACT_SILU_GLU the same without the one: silu(g) u for limit = +inf and alpha = 1
+__device__ __forceinline__ float gated_act(float g, float u, float limit, float alpha, int act) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + __expf(-alpha * g)) * (u + (act == SM_ACT_SILU_GLU ? 0.f : 1.f));
+}
+__device__ __forceinline__ bool act_is_gated(int act) { return act == SM_ACT_CLAMPED_GLU || act == SM_ACT_SILU_GLU; }
 __device__ __forceinline__ float plain_act(float z, int act) { return act == SM_ACT_GELU_TANH ? gelu_tanh(z) : gelu_erf(z); }
 
 static inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }

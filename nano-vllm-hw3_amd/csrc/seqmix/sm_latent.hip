@@ -11,7 +11,7 @@ __global__ __launch_bounds__(64) void latent_norm_store_kernel(const T* __restri
                                                                const T* __restrict__ w, float eps, T* __restrict__ cache,
                                                                const int32_t* __restrict__ slot_mapping, int R) {
     const int64_t t = blockIdx.x;
-    const int slot = slot_mapping[t];
+    const int64_t slot = slot_mapping ? slot_mapping[t] : t;        // no mapping: a dense result, row by row
     if (slot < 0) return;
     const T* xr = x + (size_t)t * row_stride;
     float ss = 0.f;
@@ -160,6 +160,20 @@ extern "C" int sm_latent_norm_store(int dtype, const void* x, int64_t row_stride
                 hipLaunchKernelGGL(latent_norm_store_kernel<DT>, dim3((unsigned)T), dim3(64), 0, as_stream(stream), (const DT*)x,
                                    row_stride, (const DT*)w, eps, (DT*)cache, slot_mapping, R));
     SM_CHECK_LAUNCH("sm_latent_norm_store");
+    return SM_OK;
+}
+
+extern "C" int sm_rms_norm_rows(int dtype, const void* x, int64_t row_stride, const void* w, float eps, void* out, int64_t T,
+                                int R, void* stream) {
+    if (T < 0 || R < 1 || row_stride < R || (T > 0 && (!x || !w || !out))) {
+        set_error("sm_rms_norm_rows: bad argument");
+        return SM_EINVAL;
+    }
+    if (T == 0) return SM_OK;
+    SM_DISPATCH(dtype, "sm_rms_norm_rows",
+                hipLaunchKernelGGL(latent_norm_store_kernel<DT>, dim3((unsigned)T), dim3(64), 0, as_stream(stream), (const DT*)x,
+                                   row_stride, (const DT*)w, eps, (DT*)out, (const int32_t*)nullptr, R));
+    SM_CHECK_LAUNCH("sm_rms_norm_rows");
     return SM_OK;
 }
 

@@ -14,7 +14,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
                                                         int32_t* __restrict__ idx, float* __restrict__ wts, int64_t T_all, int W,
                                                         int E, int top, int groups, int keep, int score,
                                                         const float* __restrict__ correction, int group_top, int renorm,
-                                                        int staged) {
+                                                        int staged, const float* __restrict__ bias) {
     extern __shared__ float z_all[];             // per token: E scores, then `groups` group scores; then the staged rows
     const int64_t t0 = (int64_t)blockIdx.x * kRouteTokens;
     const int nt = (int)min((int64_t)kRouteTokens, T_all - t0);
@@ -66,6 +66,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     // one thread finishes a token: E is small and the selections are sequential by nature
     const int64_t t = t0 + threadIdx.x;
     float* z = z_all + threadIdx.x * (E + groups);
+    if (bias != nullptr)
+        for (int e = 0; e < E; ++e) z[e] += bias[e];
     if (score == SM_ROUTE_SIGMOID) {
         for (int e = 0; e < E; ++e) z[e] = 1.f / (1.f + expf(-z[e]));
     } else {
@@ -171,12 +173,6 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     }
 }
 
-__device__ __forceinline__ float clamped_glu(float g, float u, float limit, float alpha) {
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-    return g / (1.f + __expf(-alpha * g)) * (u + 1.f);
-}
-
 // workgroup = one (token, expert) pair; every wave produces outputs f = wave, wave + 4, ...
 template <typename T>
 __global__ __launch_bounds__(256) void moe_pairs_gate_up_kernel(const T* __restrict__ h, const int32_t* __restrict__ idx,
@@ -188,7 +184,7 @@ __global__ __launch_bounds__(256) void moe_pairs_gate_up_kernel(const T* __restr
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int c = threadIdx.x; c < W; c += 256) h_lds[c] = to_f(h[(size_t)t * W + c]);
     __syncthreads();
-    if (act_kind != SM_ACT_CLAMPED_GLU) {            // one product per expert: w_gu is [E, F, W]
+    if (!act_is_gated(act_kind)) {                   // one product per expert: w_gu is [E, F, W]
         const T* wu = w_gu + (size_t)e * F * W;
         for (int f = wave; f < F; f += 4) {
             const T* u_row = wu + (size_t)f * W;
@@ -212,7 +208,7 @@ __global__ __launch_bounds__(256) void moe_pairs_gate_up_kernel(const T* __restr
         g = wave_sum(g);
         u = wave_sum(u);
         // the products leave the matrix unit in the storage type, as a GEMM's output would
-        if (lane == 0) act[(size_t)p * F + f] = from_f<T>(clamped_glu(to_f(from_f<T>(g)), to_f(from_f<T>(u)), limit, alpha));
+        if (lane == 0) act[(size_t)p * F + f] = from_f<T>(gated_act(to_f(from_f<T>(g)), to_f(from_f<T>(u)), limit, alpha, act_kind));
     }
 }
 
@@ -257,7 +253,7 @@ using namespace sm;
 
 extern "C" int sm_moe_route(int dtype, const void* h, const float* router_w, int32_t* idx, float* wts, int64_t T, int W, int E,
                             int top, int groups, int keep, int score, const float* correction, int group_top, int renorm,
-                            void* stream) {
+                            const float* bias, void* stream) {
     if (T < 0 || W < 1 || E < 1 || top < 1 || (score != SM_ROUTE_SOFTMAX && score != SM_ROUTE_SIGMOID) || group_top < 1 ||
         group_top > 4 || (T > 0 && (!h || !router_w || !idx || !wts))) {
         set_error("sm_moe_route: bad argument");
@@ -276,14 +272,14 @@ extern "C" int sm_moe_route(int dtype, const void* h, const float* router_w, int
     SM_DISPATCH(dtype, "sm_moe_route",
                 hipLaunchKernelGGL(moe_route_kernel<DT>, dim3((unsigned)((T + kRouteTokens - 1) / kRouteTokens)), dim3(256),
                                    scores + (staged ? rows : 0), as_stream(stream), (const DT*)h, router_w, idx, wts, T, W, E,
-                                   top, groups, keep, score, correction, group_top, renorm, staged));
+                                   top, groups, keep, score, correction, group_top, renorm, staged, bias));
     SM_CHECK_LAUNCH("sm_moe_route");
     return SM_OK;
 }
 
 extern "C" int sm_moe_pairs_gate_up(int dtype, const void* h, const int32_t* idx, const void* w_gu, float limit, float alpha,
                                     int act_kind, void* act, int64_t T, int top, int W, int F, void* stream) {
-    if (T < 0 || top < 1 || W < 1 || F < 1 || act_kind < 0 || act_kind > SM_ACT_GELU_TANH || (T > 0 && (!h || !idx || !w_gu || !act))) {
+    if (T < 0 || top < 1 || W < 1 || F < 1 || act_kind < 0 || act_kind > SM_ACT_SILU_GLU || (T > 0 && (!h || !idx || !w_gu || !act))) {
         set_error("sm_moe_pairs_gate_up: bad argument");
         return SM_EINVAL;
     }

@@ -46,12 +46,9 @@ __global__ __launch_bounds__(1024) void moe_align_kernel(const int32_t* __restri
     }
 }
 
-__device__ __forceinline__ float glu_bf16(float g, float u, float limit, float alpha) {
-    g = (float)(bf16_t)g;                        // the products leave the matrix unit in bf16, as a GEMM's output would
-    u = (float)(bf16_t)u;
-    g = fminf(g, limit);
-    u = fminf(fmaxf(u, -limit), limit);
-    return g / (1.f + __expf(-alpha * g)) * (u + 1.f);
+__device__ __forceinline__ float glu_bf16(float g, float u, float limit, float alpha, int act) {
+    // the products leave the matrix unit in bf16, as a GEMM's output would
+    return gated_act((float)(bf16_t)g, (float)(bf16_t)u, limit, alpha, act);
 }
 
 __device__ __forceinline__ bf16x8 load8(const unsigned short* p, int k, int K) {
@@ -62,7 +59,7 @@ __device__ __forceinline__ bf16x8 load8(const unsigned short* p, int k, int K) {
 
 // GATE_UP: A = h rows gathered by token, B = the expert's gate and up rows, out = act [rows, N] (N = F, K = W)
 // else:    A = act rows,                 B = the expert's down rows,       out = per-row products [rows, N] (N = W, K = F)
-// MODE 0: the down product; 1: gate and up with the clamped GLU; 2: the up product alone with a GELU (act_kind)
+// MODE 0: the down product; 1: gate and up with the gated activation (act_kind: clamped GLU or silu(g) u); 2: the up product alone with a GELU (act_kind)
 template <int MODE>
 __global__ __launch_bounds__(256) void moe_grouped_kernel(const unsigned short* __restrict__ a, const unsigned short* __restrict__ w,
                                                           const int32_t* __restrict__ row_pair, const int32_t* __restrict__ tile_expert,
@@ -124,7 +121,7 @@ __global__ __launch_bounds__(256) void moe_grouped_kernel(const unsigned short* 
     for (int r = 0; r < 16; ++r) {
         const int orow = tile * kRowsPerTile + (r & 3) + 8 * (r >> 2) + 4 * hi;
         if (row_pair[orow] < 0) continue;
-        const float v = GATE_UP ? glu_bf16(acc[r], acc2[r], limit, alpha) : (MODE == 2 ? plain_act((float)(bf16_t)acc[r], act_kind) : acc[r]);
+        const float v = GATE_UP ? glu_bf16(acc[r], acc2[r], limit, alpha, act_kind) : (MODE == 2 ? plain_act((float)(bf16_t)acc[r], act_kind) : acc[r]);
         out[(size_t)orow * N + n0 + l31] = __builtin_bit_cast(unsigned short, (bf16_t)v);
     }
 }
@@ -156,7 +153,7 @@ extern "C" int sm_moe_grouped_tiles(int64_t T, int top, int E) {
 extern "C" int sm_moe_grouped(const void* h, const int32_t* idx, const float* wts, const void* w_gu, const void* w_down,
                               const void* shared, float limit, float alpha, int act_kind, void* y, int64_t T, int top, int E, int W, int F,
                               int32_t* row_pair, int32_t* tile_expert, int32_t* pair_row, void* act, void* prod, void* stream) {
-    if (T < 0 || top < 1 || E < 1 || W < 1 || F < 1 || act_kind < 0 || act_kind > SM_ACT_GELU_TANH ||
+    if (T < 0 || top < 1 || E < 1 || W < 1 || F < 1 || act_kind < 0 || act_kind > SM_ACT_SILU_GLU ||
         (T > 0 && (!h || !idx || !wts || !w_gu || !w_down || !y || !row_pair || !tile_expert || !pair_row || !act || !prod))) {
         set_error("sm_moe_grouped: bad argument");
         return SM_EINVAL;
@@ -171,7 +168,7 @@ extern "C" int sm_moe_grouped(const void* h, const int32_t* idx, const float* wt
     hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)3 * E * sizeof(int), s, idx, (int)(T * top), E, tiles, row_pair,
                        tile_expert, pair_row);
     SM_CHECK_LAUNCH("sm_moe_grouped (align)");
-    if (act_kind == SM_ACT_CLAMPED_GLU)
+    if (act_kind == SM_ACT_CLAMPED_GLU || act_kind == SM_ACT_SILU_GLU)
         hipLaunchKernelGGL(moe_grouped_kernel<1>, dim3((unsigned)tiles, (unsigned)((F + 127) / 128)), dim3(256), 0, s,
                            (const unsigned short*)h, (const unsigned short*)w_gu, row_pair, tile_expert, (unsigned short*)act, top, F,
                            W, limit, alpha, act_kind);

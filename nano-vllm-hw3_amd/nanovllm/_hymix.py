@@ -24,15 +24,18 @@ SIGNATURES = {
                                  _int, _vp]),
     "hm_token_shift": (_int, [_int, _vp, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _int, _vp]),
     "hm_qkv_prepare": (_int, [_int, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _f, _vp, _int, _int, _vp, _vp, _vp, _vp, _vp,
-                              _i64, _vp, _vp, _i64, _vp, _vp, _vp, _vp]),
+                              _i64, _vp, _vp, _i64, _vp, _vp, _vp, _int, _f, _int, _vp]),
     "hm_attn_rows": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _f, _vp, _i64, _int, _int, _int, _int, _int,
-                            _int, _vp, _vp, _int, _int, _vp]),
+                            _int, _vp, _vp, _int, _int, _int, _vp, _int, _vp]),
     "hm_pool_blocks": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int, _int, _int, _int, _int, _int, _vp]),
     "hm_attn_tiles": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _f, _vp, _int, _int, _int, _int, _int, _int, _int, _int,
-                             _vp, _vp, _int, _int, _vp]),
+                             _vp, _vp, _int, _int, _int, _vp, _int, _vp]),
     "hm_attn_decode_workspace_bytes": (_sz, [_i64, _int, _int, _int]),
     "hm_attn_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _f, _vp, _i64, _int, _int, _int, _int, _int, _int, _int,
-                              _vp, _sz, _vp, _vp, _int, _int, _vp]),
+                              _vp, _sz, _vp, _vp, _int, _int, _int, _vp, _int, _vp]),
+    "hm_lightning_recurrence": (_int, [_int, _vp, _i64, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _vp, _int, _int, _int, _int,
+                                       _int, _vp]),
+    "hm_dyt_residual": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _vp]),
     "hm_group_norm_residual": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _int, _f, _vp, _i64, _int, _vp]),
     "hm_scale_softcap": (_int, [_vp, _i64, _f, _f, _vp]),
     "hm_delta_prepare": (_int, [_int, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp, _int, _f, _f, _vp, _i64, _int, _int, _vp]),

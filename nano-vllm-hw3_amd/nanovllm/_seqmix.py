@@ -23,6 +23,7 @@ SIGNATURES = {
     "sm_canon_conv": (_int, [_int, _vp, _vp, _vp, _int, _int, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _vp]),
     "sm_canon_update": (_int, [_int, _vp, _vp, _int, _int, _vp, _vp, _int, _int, _int, _vp]),
     "sm_latent_norm_store": (_int, [_int, _vp, _i64, _vp, _f, _vp, _vp, _i64, _int, _vp]),
+    "sm_rms_norm_rows": (_int, [_int, _vp, _i64, _vp, _f, _vp, _i64, _int, _vp]),
     "sm_latent_attn_rows": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _f, _i64, _int, _int, _int, _int, _int, _int, _vp]),
     "sm_latent_rope_store": (_int, [_int, _vp, _i64, _vp, _f, _vp, _i64, _vp, _vp, _int, _vp, _vp, _vp, _i64, _int, _int, _int,
                                     _int, _vp]),
@@ -31,7 +32,7 @@ SIGNATURES = {
     "sm_latent_attn_decode": (_int, [_vp, _vp, _vp, _vp, _vp, _f, _i64, _int, _int, _int, _int, _int, _vp, _sz, _int, _int, _vp]),
     "sm_poly_norm": (_int, [_int, _vp, _vp, _f, _vp, _i64, _int, _vp]),
     "sm_clamped_glu": (_int, [_int, _vp, _f, _f, _vp, _i64, _int, _vp]),
-    "sm_moe_route": (_int, [_int, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _int, _int, _int, _vp, _int, _int, _vp]),
+    "sm_moe_route": (_int, [_int, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _int, _int, _int, _vp, _int, _int, _vp, _vp]),
     "sm_moe_pairs_gate_up": (_int, [_int, _vp, _vp, _vp, _f, _f, _int, _vp, _i64, _int, _int, _int, _vp]),
     "sm_moe_pairs_down": (_int, [_int, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int, _vp]),
     "sm_moe_grouped_tiles": (_int, [_i64, _int, _int]),

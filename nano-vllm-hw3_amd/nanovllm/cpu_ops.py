@@ -145,6 +145,11 @@ def rotate_pairs(x, pos, inv_freq, rot_dims):
     return out
 
 
+def rms_norm_rows(x, w, eps):
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(x.dtype)
+
+
 def latent_rope_store(x, w, eps, q, qa, inv_freq, rot_dims, H, D, R, Rd, cache, ctx):
     T = x.shape[0]
     xf = x.float()
@@ -196,9 +201,11 @@ def clamped_glu(gu, limit, alpha):
     return (g * torch.sigmoid(alpha * g) * (u + 1)).to(gu.dtype)
 
 
-def moe_route(h, router_w, top, groups, keep, score=0, correction=None, group_top=1, renorm=True):
+def moe_route(h, router_w, top, groups, keep, score=0, correction=None, group_top=1, renorm=True, bias=None):
     T, E = h.shape[0], router_w.shape[0]
     z = h.float() @ router_w.t()
+    if bias is not None:
+        z = z + bias.float()
     s = torch.sigmoid(z) if score == 1 else torch.softmax(z, -1)
     choice = s if correction is None else s + correction.float()
     masked = choice
@@ -218,6 +225,10 @@ def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared, act_kind=0):
         tok, k = (idx == e).nonzero(as_tuple=True)
         if act_kind == 0:
             act = clamped_glu(F.linear(h[tok], w_gu[e]), limit, alpha)
+        elif act_kind == 3:
+            g, u = F.linear(h[tok], w_gu[e]).float().chunk(2, -1)
+            g, u = g.clamp(max=limit), u.clamp(-limit, limit)
+            act = (g * torch.sigmoid(alpha * g) * u).to(h.dtype)
         else:
             act = F.gelu(F.linear(h[tok], w_gu[e]).float(), approximate="tanh" if act_kind == 2 else "none").to(h.dtype)
         y.index_add_(0, tok, wts[tok, k][:, None] * F.linear(act, w_down[e]).float())
@@ -258,18 +269,37 @@ def token_shift(h, mu, state, layer, ctx):
     return (hf + (prev - hf) * mu.float()).to(h.dtype)
 
 
-def rotate_half_partial(x, pos, inv_freq):
-    """x f32 [T, heads, D]: the first 2 * len(inv_freq) channels of every head turn by pos * inv_freq."""
+def rotate_half_partial(x, pos, inv_freq, mag=1.0):
+    """x f32 [T, heads, D]: the first 2 * len(inv_freq) channels of every head turn by pos * inv_freq (cosines and sines
+    times ``mag``)."""
     half = inv_freq.numel()
     ang = pos.float()[:, None] * inv_freq[None, :]
-    c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    c, s = (torch.cos(ang) * mag)[:, None, :], (torch.sin(ang) * mag)[:, None, :]
     a, b = x[..., :half], x[..., half:2 * half]
     return torch.cat([a * c - b * s, b * c + a * s, x[..., 2 * half:]], -1)
 
 
+def rotate_pairs_partial(x, pos, inv_freq, mag):
+    """x f32 [T, heads, D]: channels (2i, 2i + 1), i < len(inv_freq), of every head turn by pos * inv_freq[i]; cosines and
+    sines times ``mag``."""
+    n = inv_freq.numel()
+    ang = pos.float()[:, None] * inv_freq[None, :]
+    c, s = (torch.cos(ang) * mag)[:, None, :], (torch.sin(ang) * mag)[:, None, :]
+    a, b = x[..., 0:2 * n:2], x[..., 1:2 * n:2]
+    out = x.clone()
+    out[..., 0:2 * n:2] = a * c - b * s
+    out[..., 1:2 * n:2] = b * c + a * s
+    return out
+
+
 def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, ctx, k_cache, v_cache, v_first, lam,
-                q_head_w=None, k_head_w=None, q_head_scale=None):
+                q_head_w=None, k_head_w=None, q_head_scale=None, interleaved=False, rot_mag=1.0, v_unit_norm=False):
     T = qkv.shape[0]
+
+    def turn(x):                                        # (the pairing this call asks for)
+        if interleaved:
+            return rotate_pairs_partial(x, ctx.tok_pos, inv_freq, rot_mag)
+        return rotate_half_partial(x, ctx.tok_pos, inv_freq, rot_mag)
     if k_cache is None:                        # the rows hold q only
         q = qkv.float().reshape(T, H, D)
         if q_head_w is not None:
@@ -277,7 +307,7 @@ def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, c
         if q_head_scale is not None:
             q = q * q_head_scale.float()[None, :, None]
         if inv_freq is not None:
-            q = rotate_half_partial(q, ctx.tok_pos, inv_freq)
+            q = turn(q)
         if unit_norm:
             q = _unit_rms(q, eps)
         return q.to(qkv.dtype).contiguous()
@@ -290,11 +320,13 @@ def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, c
     if q_head_scale is not None:
         q = q * q_head_scale.float()[None, :, None]
     if inv_freq is not None:
-        q, k = rotate_half_partial(q, ctx.tok_pos, inv_freq), rotate_half_partial(k, ctx.tok_pos, inv_freq)
+        q, k = turn(q), turn(k)
     if unit_norm:
         q, k = _unit_rms(q, eps), _unit_rms(k, eps)
     if v_first is not None:
         v = (1 - lam.float()) * v + lam.float() * v_first.float()
+    if v_unit_norm:
+        v = _unit_rms(v.reshape(T, G, V), eps).reshape(T, G * V)
     rows = ctx.slot_mapping.long()
     k_cache.view(-1, G, D)[rows] = k.to(k_cache.dtype)
     v_cache.view(-1, G, V)[rows] = v.reshape(T, G, V).to(v_cache.dtype)
@@ -317,7 +349,8 @@ def pool_blocks(k_cache, v_cache, kp_cache, vp_cache, pool, ctx):
         vp[prow] = vr[rows].float().mean(0).to(vp.dtype)
 
 
-def paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first, pooled=None):
+def paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first, pooled=None, chunk=0, sigmoid=False,
+                    head_bias=None):
     T, H, D = q.shape
     bs, G, V = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     o = torch.empty((T, H * V), dtype=q.dtype)
@@ -337,6 +370,13 @@ def paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first, p
         ok = j[None, :] <= i
         if window > 0:
             ok &= ((i - j[None, :]) < window) | (j[None, :] < keep_first)
+        if chunk > 0:
+            ok &= (i // chunk) == (j[None, :] // chunk)
+        if sigmoid:
+            hb = head_bias.float()[None, :, None] if head_bias is not None else 0.0
+            p = torch.sigmoid(s + hb) * ok[:, None, :]
+            o[a:e] = torch.einsum("thn,nhv->thv", p, vv).reshape(e - a, H * V).to(q.dtype)
+            continue
         s = s.masked_fill(~ok[:, None, :], float("-inf"))
         if pooled is not None and pooled[2] > 0:
             kp_c, vp_c, pool = pooled
@@ -422,3 +462,39 @@ def scale_softcap_(logits, scale, cap):
     if cap:
         logits.copy_(cap * torch.tanh(logits / cap))
     return logits
+
+
+def dyt_residual(x, y, post, nxt, dtype, ids, want_h):
+    def dyt(v, n):
+        w, b, a = n
+        return torch.tanh(a.float() * v) * w.float() + b.float()
+    if y is not None:
+        if ids is not None:
+            x = y[ids].float()
+        else:
+            x += dyt(y.float(), post)
+    if not want_h:
+        return x, None
+    h = dyt(x, nxt).to(dtype) if nxt is not None else (x if dtype == torch.float32 else x.to(dtype))
+    return x, h
+
+
+def lightning_recurrence(proj, q_off, k_off, v_off, H, D, V, decay, state, ctx):
+    T = proj.shape[0]
+    pf = proj.float()
+    q = F.silu(pf[:, q_off:q_off + H * D]).reshape(T, H, D)
+    k = F.silu(pf[:, k_off:k_off + H * D]).reshape(T, H, D)
+    v = F.silu(pf[:, v_off:v_off + H * V]).reshape(T, H, V)
+    o = torch.empty((T, H, V), dtype=torch.float32)
+    qs = ctx.qstart.tolist()
+    for b in range(ctx.num_seqs):
+        a, e = qs[b], qs[b + 1]
+        if e <= a:
+            continue
+        slot = int(ctx.seq_slot[b])
+        S = state[slot].clone() if int(ctx.seq_pos0[b]) > 0 else torch.zeros_like(state[slot])
+        for t in range(a, e):
+            S = decay.float()[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[slot] = S
+    return o

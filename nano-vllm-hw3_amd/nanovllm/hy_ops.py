@@ -83,8 +83,33 @@ def rotary_inv_freq(dims, base, device):
     return (float(base) ** (-2.0 * i / dims)).to(torch.float32).to(device)
 
 
+def rotary_table(dims, base, device, scaling=None):
+    """(frequencies f32 [dims/2], factor on every cosine and sine).  Without ``scaling``: f_i = base^(-2i/dims) and 1.
+    ``scaling`` = {factor, original, fast, slow} stretches the table for contexts longer than ``original`` positions: a
+    pair that makes fewer than ``slow`` turns over ``original`` positions has its frequency divided by ``factor``, one that
+    makes more than ``fast`` turns keeps it, and between them a linear ramp over the pair index blends the two (the ramp
+    runs from pair lo = floor(d(fast)) to hi = ceil(d(slow)), d(t) = dims ln(original / (2 pi t)) / (2 ln base), clamped
+    to the table); cosines and sines grow by 0.1 ln(factor) + 1.  Evaluated in float64, kept in float32."""
+    import math
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    mag = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def pair_of(turns):
+            return dims * math.log(orig / (2 * math.pi * turns)) / (2 * math.log(float(base)))
+        lo = max(math.floor(pair_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(pair_of(float(scaling["slow"]))), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    return f.to(torch.float32).to(device), mag
+
+
 def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, ctx: StepContext, k_cache, v_cache,
-                v_first=None, lam=None, q_head_w=None, k_head_w=None, q_head_scale=None):
+                v_first=None, lam=None, q_head_w=None, k_head_w=None, q_head_scale=None, interleaved=False, rot_mag=1.0,
+                v_unit_norm=False):
     """From the merged product qkv [T, H*D + G*D + G*V] of a step's tokens, in one launch per token:
       q_norm_w / k_norm_w given: RMS norm over the WHOLE q (k) projection with that weight;
       rotation of the first 2 * len(inv_freq) channels of every q and k head by position * inv_freq (channel i paired
@@ -94,10 +119,12 @@ def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, c
       k and v are stored at the tokens' cache rows; returns q [T, H, D].
     q_head_w / k_head_w [D]: before the rotation every q (k) head is divided by its own RMS and multiplied by that row,
     shared by the heads; q_head_scale f32 [H]: query head h times its number after that.  inv_freq None: no rotation.
-    k_cache None: qkv holds q only [T, H*D] (the layer reads another layer's keys and values); nothing is stored."""
+    k_cache None: qkv holds q only [T, H*D] (the layer reads another layer's keys and values); nothing is stored.
+    interleaved: channel 2i pairs with 2i + 1 instead; rot_mag multiplies every cosine and sine; v_unit_norm: every value
+    head is divided by its RMS (no weight) before it is stored."""
     if not qkv.is_cuda:
         return cpu_ops.qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, ctx, k_cache, v_cache,
-                                   v_first, lam, q_head_w, k_head_w, q_head_scale)
+                                   v_first, lam, q_head_w, k_head_w, q_head_scale, interleaved, rot_mag, v_unit_norm)
     _rows(qkv, "qkv")
     T = qkv.shape[0]
     if k_cache is None:
@@ -115,7 +142,8 @@ def qkv_prepare(qkv, H, G, D, V, q_norm_w, k_norm_w, eps, inv_freq, unit_norm, c
                                       HM.ptr(k_norm_w), float(eps), HM.ptr(inv_freq), inv_freq.numel() if inv_freq is not None else 0,
                                       int(bool(unit_norm)), ctx.tok_pos.data_ptr(), ctx.slot_mapping.data_ptr(), HM.ptr(k_cache),
                                       HM.ptr(v_cache), HM.ptr(v_first), v_first.stride(0) if v_first is not None else 0, HM.ptr(lam),
-                                      q.data_ptr(), T, HM.ptr(q_head_w), HM.ptr(k_head_w), HM.ptr(q_head_scale), _dev(qkv)))
+                                      q.data_ptr(), T, HM.ptr(q_head_w), HM.ptr(k_head_w), HM.ptr(q_head_scale),
+                                      int(bool(interleaved)), float(rot_mag), int(bool(v_unit_norm)), _dev(qkv)))
     return q
 
 
@@ -144,19 +172,24 @@ USE_TILES = True       # bf16 attention on the matrix cores where the shape allo
 
 
 def paged_attention(q, k_cache, v_cache, ctx: StepContext, scale, sink=None, window=0, keep_first=0, force_rows=False,
-                    pooled=None):
+                    pooled=None, chunk=0, sigmoid=False, head_bias=None):
     """q [T, H, D] over the paged caches k [blocks, block_size, G, D], v [blocks, block_size, G, V]; query head h reads
     key/value head h // (H/G).  The token at position i sees key j <= i, and with window > 0 only if i - j < window or
     j < keep_first.  ``sink`` f32 [H]: one more term exp(sink[h]) in the softmax denominator, without a value (zeros
     = a sink of score 0).  Scores and weights are float32.  Returns [T, H * V].
     ``pooled`` = (kp_cache, vp_cache, pool) with window > 0: beside its window the token also sees one key and value for
     every block of ``pool`` tokens whose last token lies at or before i - window (the block means pool_blocks keeps), in the
-    same softmax."""
+    same softmax.
+    ``chunk`` > 0: the token at position i sees key j <= i only if i // chunk == j // chunk (chunks of positions counted from
+    the sequence's start).  ``sigmoid``: the weight of a visible key is sigmoid(score + head_bias[h]) (f32 [H], None = 0),
+    not normalised over the keys."""
     if not q.is_cuda:
-        return cpu_ops.paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first, pooled)
+        return cpu_ops.paged_attention(q, k_cache, v_cache, ctx, scale, sink, window, keep_first, pooled, chunk, sigmoid,
+                                       head_bias)
     kp, vp, pool = pooled if pooled is not None else (None, None, 0)
     pr = kp.shape[1] if kp is not None else 0
-    ptail = (HM.ptr(kp), HM.ptr(vp), int(pool), int(pr))
+    ptail = (HM.ptr(kp), HM.ptr(vp), int(pool), int(pr), int(chunk), HM.ptr(head_bias), int(bool(sigmoid)))
+    assert head_bias is None or head_bias.dtype == torch.float32
     HM.require_cuda(q, k_cache.dtype, "q")
     T, H, D = q.shape
     bs, G, V = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
@@ -167,6 +200,8 @@ def paged_attention(q, k_cache, v_cache, ctx: StepContext, scale, sink=None, win
                 V <= 128 and bs % 64 == 0)
     if tiles_ok and ctx.max_q == 1 and H // G <= 32:
         keys = min(mb * bs, window + keep_first + 128) if window > 0 else mb * bs
+        if chunk > 0:
+            keys = min(keys, chunk + 64)
         if pool:
             keys = min(mb * bs, keys + mb * bs // pool + 64)
         splits = decode_splits(ctx.num_seqs * G, keys)
@@ -284,3 +319,49 @@ def relu_squared(z):
     out = torch.empty((T, Fw), dtype=z.dtype, device=z.device)
     HM.check(HM.load().hm_relu_squared(HM.dtype_code(z.dtype), z.data_ptr(), z.stride(0), out.data_ptr(), T, Fw, _dev(z)))
     return out
+
+
+def dyt_residual(x, y, post, nxt, dtype, ids=None, want_h=True):
+    """The boundary between two sublayers of a float32 residual x [T, W] whose sublayers sit between two Dynamic-Tanh
+    norms, dyt(z) = tanh(alpha z) * w + b with a norm given as (w [W], b [W], alpha f32 [1]); one elementwise launch:
+      y given:   x <- x + dyt_post(y)     (ids given: x <- y[ids], y an embedding table, no norm; x may be None)
+      want_h:    returns dyt_nxt(x), or x itself without ``nxt``, in ``dtype``.
+    Returns (x, h)."""
+    src = y if y is not None else x
+    if not src.is_cuda:
+        return cpu_ops.dyt_residual(x, y, post, nxt, dtype, ids, want_h)
+    T = ids.numel() if ids is not None else src.shape[0]
+    W = src.shape[1]
+    if x is None:
+        x = torch.empty((T, W), dtype=torch.float32, device=src.device)
+    if y is not None:
+        HM.require_cuda(y, dtype, "y")
+    pw, pb, pa = post if post is not None else (None, None, None)
+    nw, nb, na = nxt if nxt is not None else (None, None, None)
+    for a in (pa, na):
+        assert a is None or a.dtype == torch.float32
+    h = None
+    if want_h and (nxt is not None or dtype != torch.float32):
+        h = torch.empty((T, W), dtype=dtype, device=x.device)
+    HM.check(HM.load().hm_dyt_residual(HM.dtype_code(dtype), x.data_ptr(), HM.ptr(y), HM.ptr(ids), HM.ptr(pw), HM.ptr(pb), HM.ptr(pa),
+                                       HM.ptr(nw), HM.ptr(nb), HM.ptr(na), HM.ptr(h), T, W, _dev(x)))
+    return x, (h if h is not None or not want_h else x)
+
+
+def lightning_recurrence(proj, q_off, k_off, v_off, H, D, V, decay, state, ctx: StepContext):
+    """Linear attention with a constant decay per head over every sequence's portion, token after token, with a float32
+    state S [D, V] per head:  S <- decay[h] S + k v^T,  o = S^T q,  where q, k [T, H*D] and v [T, H*V] are silu of the
+    columns q_off, k_off, v_off of proj.  state f32 [slots, H, D, V] is read at a portion's start (zero at position 0) and
+    left at its end.  decay f32 [H].  Returns o f32 [T, H, V]."""
+    if not proj.is_cuda:
+        return cpu_ops.lightning_recurrence(proj, q_off, k_off, v_off, H, D, V, decay, state, ctx)
+    _rows(proj, "proj")
+    T = proj.shape[0]
+    assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, D, V)
+    assert decay.dtype == torch.float32 and decay.numel() == H
+    o = torch.empty((T, H, V), dtype=torch.float32, device=proj.device)
+    HM.check(HM.load().hm_lightning_recurrence(HM.dtype_code(proj.dtype), proj.data_ptr(), proj.stride(0), q_off, k_off, v_off,
+                                               decay.data_ptr(), state.data_ptr(), ctx.qstart.data_ptr(), ctx.seq_pos0.data_ptr(),
+                                               ctx.seq_slot.data_ptr(), o.data_ptr(), ctx.num_seqs, H, D, V,
+                                               max(int(ctx.max_q), 1), _dev(proj)))
+    return o

@@ -42,18 +42,24 @@ class RoutedExperts(nn.Module):
     Variations: ``score`` = "sigmoid" (independent scores instead of a softmax); ``correction``: a learned per-expert
     number added to the scores for the CHOICE of groups and experts only (the weights stay the scores); ``group_top``: a
     group scores the sum of that many of its largest choice scores instead of the largest; ``renorm`` = False: the chosen
-    scores weigh as they are; ``act`` = "gelu" / "gelu_tanh": an expert is down(gelu(up h)), no gate, no clamp."""
+    scores weigh as they are; ``act`` = "gelu" / "gelu_tanh": an expert is down(gelu(up h)), no gate, no clamp;
+    ``act`` = "silu_glu": an expert is down(silu(gate h) * up h), no clamp; ``bias``: a learned number per expert added to
+    the router's logits (with softmax scores and ``renorm`` the weights are the softmax over the chosen logits)."""
 
-    ACTS = {"clamped_glu": seq_ops.ACT_CLAMPED_GLU, "gelu": seq_ops.ACT_GELU, "gelu_tanh": seq_ops.ACT_GELU_TANH}
+    ACTS = {"clamped_glu": seq_ops.ACT_CLAMPED_GLU, "gelu": seq_ops.ACT_GELU, "gelu_tanh": seq_ops.ACT_GELU_TANH,
+            "silu_glu": seq_ops.ACT_SILU_GLU}
 
     def __init__(self, width: int, experts: int, top: int, ff: int, limit: float = 0.0, groups: int = 1, keep: int = 1,
                  shared: ClampedGLU = None, alpha: float = 1.702, score: str = "softmax", correction: bool = False,
-                 group_top: int = 1, renorm: bool = True, act: str = "clamped_glu"):
+                 group_top: int = 1, renorm: bool = True, act: str = "clamped_glu", bias: bool = False):
         super().__init__()
+        if act == "silu_glu":                  # the gated form with nothing clamped and a plain sigmoid
+            limit, alpha = float("inf"), 1.0
         self.experts, self.top, self.groups, self.keep, self.limit, self.alpha = experts, top, groups, keep, float(limit), alpha
         self.score = {"softmax": seq_ops.ROUTE_SOFTMAX, "sigmoid": seq_ops.ROUTE_SIGMOID}[score]
         self.group_top, self.renorm, self.act_kind = group_top, renorm, self.ACTS[act]
-        self.parts = 2 if act == "clamped_glu" else 1           # gate and up rows, or up rows alone
+        self.parts = 2 if self.act_kind in seq_ops.GATED_ACTS else 1           # gate and up rows, or up rows alone
+        self.bias = nn.Parameter(torch.zeros(experts, dtype=torch.float32), requires_grad=False) if bias else None
         self.correction = nn.Parameter(torch.zeros(experts, dtype=torch.float32), requires_grad=False) if correction else None
         self.router = nn.Parameter(torch.empty(experts, width, dtype=torch.float32), requires_grad=False)
         self.w_gu = nn.Parameter(torch.empty(experts, self.parts * ff, width), requires_grad=False)
@@ -65,7 +71,7 @@ class RoutedExperts(nn.Module):
         if self._tiled is None and h.is_cuda and h.dtype == torch.bfloat16:
             self._tiled = (seq_ops.tile_expert_weights(self.w_gu, self.parts), seq_ops.tile_expert_weights(self.w_down))
         idx, wts = seq_ops.moe_route(h, self.router, self.top, self.groups, self.keep, self.score, self.correction,
-                                     self.group_top, self.renorm)
+                                     self.group_top, self.renorm, self.bias)
         shared = self.shared(h) if self.shared is not None else None
         return seq_ops.moe_experts(h, idx, wts, self.w_gu, self.w_down, self.limit, self.alpha, shared, tiled=self._tiled,
                                    act_kind=self.act_kind)

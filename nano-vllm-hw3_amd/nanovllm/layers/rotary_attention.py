@@ -13,6 +13,12 @@ between designs as constructor arguments:
   kv_source   another PagedRotaryAttention whose keys and values (and, for an equal ``pool``, pooled blocks) this layer
               reads: it has no k/v projection of its own, only queries, mask and output
   rot_dims    0 = positions do not enter the scores
+  interleaved the rotation pairs channel 2i with 2i + 1 instead of i with i + rot_dims / 2
+  rot_scaling {factor, original, fast, slow}: a frequency table stretched for longer contexts (hy_ops.rotary_table)
+  v_unit_norm every value head divided by its RMS (no weight) before it is cached
+  chunk       chunk > 0: a query sees a key only inside its own chunk of ``chunk`` positions (counted from position 0)
+  weights     "softmax", or "sigmoid": the weight of a visible key is sigmoid(score + b_h) with a learned number per
+              query head, not normalised over the keys
 Grouped heads: query head h reads key/value head h // (heads / kv_heads).  q, k and v come from ONE merged product."""
 import torch
 import torch.nn.functional as F
@@ -23,8 +29,12 @@ from nanovllm import hy_ops, seq_ops
 
 class PagedRotaryAttention(nn.Module):
     def __init__(self, width, heads, kv_heads, dim, vdim, scale, eps, rot_dims, rot_base, proj_norm=False, unit_norm=False,
-                 sink=None, window=0, keep_first=0, v_mix=False, head_norm=False, head_temp=False, pool=0, kv_source=None):
+                 sink=None, window=0, keep_first=0, v_mix=False, head_norm=False, head_temp=False, pool=0, kv_source=None,
+                 interleaved=False, rot_scaling=None, v_unit_norm=False, chunk=0, weights="softmax"):
         super().__init__()
+        assert weights in ("softmax", "sigmoid") and not (weights == "sigmoid" and (sink or pool))
+        assert not chunk or (not keep_first and not pool), "a chunked mask goes without kept first tokens and pooled blocks"
+        assert not (v_unit_norm and (v_mix or kv_source is not None))
         assert heads % kv_heads == 0 and rot_dims % 2 == 0 and rot_dims <= dim and sink in (None, "learned", "zero")
         assert not pool or (window > 0 and not keep_first), "pooled blocks go with a window that keeps no first tokens"
         assert kv_source is None or (kv_source.kv_heads, kv_source.dim, kv_source.vdim, kv_source.rot_dims) == \
@@ -35,6 +45,8 @@ class PagedRotaryAttention(nn.Module):
         self.window, self.keep_first, self.v_mix = int(window), int(keep_first), v_mix
         self.rot_dims, self.rot_base = rot_dims, rot_base
         self.pool = int(pool)
+        self.interleaved, self.rot_scaling, self.rot_mag = bool(interleaved), rot_scaling, 1.0
+        self.v_unit_norm, self.chunk, self.sigmoid = bool(v_unit_norm), int(chunk), weights == "sigmoid"
         self.__dict__["kv_source"] = kv_source              # (not a submodule of this layer)
         own_kv = kv_source is None
         self.qkv_proj = nn.Parameter(torch.empty(heads * dim + (kv_heads * (dim + vdim) if own_kv else 0), width),
@@ -48,6 +60,7 @@ class PagedRotaryAttention(nn.Module):
         self.q_head_norm = nn.Parameter(torch.ones(dim), requires_grad=False) if head_norm else None
         self.k_head_norm = nn.Parameter(torch.ones(dim), requires_grad=False) if head_norm and own_kv else None
         self.temp = nn.Parameter(torch.ones(heads, **f32), requires_grad=False) if head_temp else None
+        self.head_bias = nn.Parameter(torch.zeros(heads, **f32), requires_grad=False) if self.sigmoid else None
         self.inv_freq = None       # f32 [rot_dims / 2], made with the cache
         self.k_cache = self.v_cache = self.kp_cache = self.vp_cache = None
 
@@ -70,7 +83,10 @@ class PagedRotaryAttention(nn.Module):
             self.vp_cache = torch.zeros(num_blocks, rows, self.kv_heads, self.vdim, dtype=dtype, device=device)
         elif self.pool > 0:
             self.kp_cache, self.vp_cache = src.kp_cache, src.vp_cache
-        self.inv_freq = hy_ops.rotary_inv_freq(self.rot_dims, self.rot_base, device) if self.rot_dims else None
+        if self.rot_dims:
+            self.inv_freq, self.rot_mag = hy_ops.rotary_table(self.rot_dims, self.rot_base, device, self.rot_scaling)
+        else:
+            self.inv_freq = None
 
     def cache_bytes_per_token(self, itemsize, block_size=64):
         own = self.kv_heads * (self.dim + self.vdim) * itemsize
@@ -85,10 +101,10 @@ class PagedRotaryAttention(nn.Module):
         q = hy_ops.qkv_prepare(qkv, self.heads, self.kv_heads, self.dim, self.vdim, self.q_norm, self.k_norm, self.eps,
                                self.inv_freq, self.unit_norm, ctx, self.k_cache if own_kv else None,
                                self.v_cache if own_kv else None, v_first if self.v_mix else None, self.lam,
-                               self.q_head_norm, self.k_head_norm, self.temp)
+                               self.q_head_norm, self.k_head_norm, self.temp, self.interleaved, self.rot_mag, self.v_unit_norm)
         if self._pools_own():                  # the blocks this step completes (the keys are in the cache by now)
             hy_ops.pool_blocks(self.k_cache, self.v_cache, self.kp_cache, self.vp_cache, self.pool, ctx)
         pooled = (self.kp_cache, self.vp_cache, self.pool) if self.pool > 0 else None
         o = hy_ops.paged_attention(q, self.k_cache, self.v_cache, ctx, self.scale, self.sink, self.window, self.keep_first,
-                                   pooled=pooled)
+                                   pooled=pooled, chunk=self.chunk, sigmoid=self.sigmoid, head_bias=self.head_bias)
         return F.linear(o, self.o_proj), (qkv[:, (self.heads + self.kv_heads) * self.dim:] if own_kv else None)

@@ -12,6 +12,7 @@ _MODELS = {
     "Pasizen": ("nanovllm.models.pasizen", "PasizenForCausalLM"),
     "Lipelix": ("nanovllm.models.lipelix", "LipelixForCausalLM"),
     "Galupel": ("nanovllm.models.galupel", "GalupelForCausalLM"),
+    "Lilevik": ("nanovllm.models.lilevik", "LilevikForCausalLM"),
 }
 DEFAULT = "Qwen3ForCausalLM"
 

@@ -100,6 +100,18 @@ def latent_norm_store(x, w, eps, cache, slot_mapping):
                                             cache.data_ptr(), slot_mapping.data_ptr(), T, R, _dev(x)))
 
 
+def rms_norm_rows(x, w, eps):
+    """x [T, R] (rows may be a column slice of a wider product) -> x / sqrt(mean(x^2) + eps) * w, dense [T, R]."""
+    if not x.is_cuda:
+        return cpu_ops.rms_norm_rows(x, w, eps)
+    assert x.stride(1) == 1 and x.dtype == w.dtype
+    T, R = x.shape
+    out = torch.empty((T, R), dtype=x.dtype, device=x.device)
+    SM.check(SM.load().sm_rms_norm_rows(SM.dtype_code(x.dtype), x.data_ptr(), x.stride(0), w.data_ptr(), eps, out.data_ptr(), T, R,
+                                        _dev(x)))
+    return out
+
+
 def latent_rope_store(x, w, eps, q, qa, inv_freq, rot_dims, H, D, R, Rd, cache, ctx: StepContext):
     """A latent with a rotated key part.  x [T, R + Rd] (rows may be a column slice): rms_norm(x[:, :R]) * w and x[:, R:]
     with its first rot_dims channels turned by position * inv_freq (channel 2i pairs with 2i + 1) are stored as the
@@ -178,16 +190,20 @@ def clamped_glu(gu, limit, alpha=1.702):
 
 
 ROUTE_SOFTMAX, ROUTE_SIGMOID = 0, 1
-ACT_CLAMPED_GLU, ACT_GELU, ACT_GELU_TANH = 0, 1, 2
+ACT_CLAMPED_GLU, ACT_GELU, ACT_GELU_TANH, ACT_SILU_GLU = 0, 1, 2, 3
+GATED_ACTS = (ACT_CLAMPED_GLU, ACT_SILU_GLU)      # experts with gate and up rows
 
 
-def moe_route(h, router_w, top, groups=1, keep=1, score=ROUTE_SOFTMAX, correction=None, group_top=1, renorm=True):
+def moe_route(h, router_w, top, groups=1, keep=1, score=ROUTE_SOFTMAX, correction=None, group_top=1, renorm=True, bias=None):
     """Router with group-limited top-k: (idx int32 [T, top], weights f32 [T, top]); router_w f32 [E, W].  Scores are the
     softmax or the sigmoid of the float32 logits; ``correction`` f32 [E] is added for the CHOICE only (groups and
     experts), the weights stay the scores; a group scores the sum of its ``group_top`` largest choice scores (1 = its
-    maximum); ``renorm``: the chosen weights are divided by their sum."""
+    maximum); ``renorm``: the chosen weights are divided by their sum.  ``bias`` f32 [E] is added to the logits (softmax
+    scores with ``renorm`` are then the softmax over the chosen experts' logits)."""
     if not h.is_cuda:
-        return cpu_ops.moe_route(h, router_w, top, groups, keep, score, correction, group_top, renorm)
+        return cpu_ops.moe_route(h, router_w, top, groups, keep, score, correction, group_top, renorm, bias)
+    if bias is not None:
+        SM.require_cuda(bias, torch.float32, "bias")
     if correction is not None:
         SM.require_cuda(correction, torch.float32, "correction")
     SM.require_cuda(h, None, "h")
@@ -198,7 +214,7 @@ def moe_route(h, router_w, top, groups=1, keep=1, score=ROUTE_SOFTMAX, correctio
     wts = torch.empty((T, top), dtype=torch.float32, device=h.device)
     SM.check(SM.load().sm_moe_route(SM.dtype_code(h.dtype), h.data_ptr(), router_w.data_ptr(), idx.data_ptr(), wts.data_ptr(),
                                     T, W, E, top, groups, keep, int(score), SM.ptr(correction), int(group_top), int(bool(renorm)),
-                                    _dev(h)))
+                                    SM.ptr(bias), _dev(h)))
     return idx, wts
 
 
@@ -224,10 +240,11 @@ def moe_experts(h, idx, wts, w_gu, w_down, limit, alpha=1.702, shared=None, form
     forces one; by default float32 runs pair by pair and bf16 grouped by expert on the matrix cores, in tiles of 32 rows
     for small groups (decode) and of 128 rows for large ones (prefill).  ``tiled`` = (tile_expert_weights(w_gu, 2),
     tile_expert_weights(w_down)), what the grouped forms read (made here when the caller does not keep them).
-    ``act_kind`` = ACT_GELU / ACT_GELU_TANH: an expert is down(gelu(up h)) instead, w_gu is [E, F, W] (tiled in one part)."""
+    ``act_kind`` = ACT_GELU / ACT_GELU_TANH: an expert is down(gelu(up h)) instead, w_gu is [E, F, W] (tiled in one part);
+    ACT_SILU_GLU: the gated form g sigmoid(alpha g) u without the one and, with limit = inf and alpha = 1, silu(gate) * up."""
     if not h.is_cuda:
         return cpu_ops.moe_experts(h, idx, wts, w_gu, w_down, limit, alpha, shared, act_kind)
-    parts = 2 if act_kind == ACT_CLAMPED_GLU else 1
+    parts = 2 if act_kind in GATED_ACTS else 1
     assert w_gu.shape[1] == parts * w_down.shape[2]
     SM.require_cuda(h, w_gu.dtype, "h")
     T, W = h.shape
