@@ -131,8 +131,8 @@ def test_seqmix_argument_validation_needs_no_gpu():
     assert lib.sm_latent_attn_tiles(one, one, one, one, one, one, 0.1, 2, 8, 4, 64, 64, 4, 72, 0, None) == -1   # values wider than the row
     assert lib.sm_latent_rope_store(1, one, 40, one, 1e-5, one, 96, one, one, 12, one, one, one, 4, 2, 16, 32, 8, None) == -1   # rotation wider than the part
     assert lib.sm_latent_attn_decode(one, one, one, one, one, 0.1, 2, 4, 64, 64, 4, 2, one, 16, 0, 0, None) == -3   # workspace
-    assert lib.sm_moe_route(1, one, one, one, one, 4, 64, 8, 3, 4, 1, 0, None, 1, 1, None) == -2          # top > keep * E/groups
-    assert lib.sm_moe_route(1, one, one, one, one, 4, 64, 8, 2, 4, 2, 5, None, 1, 1, None) == -1          # unknown score function
+    assert lib.sm_moe_route(1, one, one, one, one, 4, 64, 8, 3, 4, 1, 0, None, 1, 1, None, None) == -2    # top > keep * E/groups
+    assert lib.sm_moe_route(1, one, one, one, one, 4, 64, 8, 2, 4, 2, 5, None, 1, 1, None, None) == -1    # unknown score function
     assert lib.sm_moe_grouped(one, one, one, one, one, None, 1.0, 1.7, 0, one, 4, 2, 8, 60, 64, one, one, one, one, one, None) == -2
     assert lib.sm_moe_grouped(one, one, one, one, one, None, 1.0, 1.7, 9, one, 4, 2, 8, 64, 64, one, one, one, one, one, None) == -1   # unknown activation
 
@@ -167,15 +167,24 @@ def test_hymix_argument_validation_needs_no_gpu():
     assert lib.hm_sublayer_close(1, one, None, None, 0, None, None, 0.5, one, 1e-5, one, None, None, 0, None, None, None, 4,
                                  1 << 20, None) == -2                                                     # wider than the row buffer
     assert lib.hm_qkv_prepare(1, one, 100, 4, 3, 16, 8, None, None, 1e-5, one, 4, 0, one, one, one, one, None, 0, None, one, 4,
-                              None, None, None, None) == -1                                               # heads % kv_heads
+                              None, None, None, 0, 1.0, 0, None) == -1                                    # heads % kv_heads
     assert lib.hm_qkv_prepare(1, one, 200, 4, 2, 16, 8, None, None, 1e-5, one, 9, 0, one, one, one, one, None, 0, None, one, 4,
-                              None, None, None, None) == -1                                               # rotation wider than a head
-    assert lib.hm_attn_tiles(one, one, one, one, one, one, None, 0, 0, 0.1, one, 2, 8, 4, 2, 20, 16, 64, 4, None, None, 0, 0, None) == -2   # dim % 8
-    assert lib.hm_attn_tiles(one, one, one, one, one, one, None, 0, 0, 0.1, one, 2, 8, 4, 2, 16, 16, 48, 4, None, None, 0, 0, None) == -2   # block % 64
-    assert lib.hm_attn_tiles(one, one, one, one, one, one, None, 0, 0, 0.1, one, 2, 8, 4, 2, 16, 16, 64, 4, one, one, 12, 6, None) == -1   # pooled blocks without a window
-    assert lib.hm_attn_rows(1, one, one, one, one, one, one, None, 40, 0, 0.1, one, 4, 4, 2, 16, 16, 64, 4, one, one, 12, 5, None) == -1   # pooled pages too small
+                              None, None, None, 1, 1.0, 0, None) == -1                                    # rotation wider than a head
+    assert lib.hm_attn_tiles(one, one, one, one, one, one, None, 0, 0, 0.1, one, 2, 8, 4, 2, 20, 16, 64, 4, None, None, 0, 0, 0, None, 0, None) == -2   # dim % 8
+    assert lib.hm_attn_tiles(one, one, one, one, one, one, None, 0, 0, 0.1, one, 2, 8, 4, 2, 16, 16, 48, 4, None, None, 0, 0, 0, None, 0, None) == -2   # block % 64
+    assert lib.hm_attn_tiles(one, one, one, one, one, one, None, 0, 0, 0.1, one, 2, 8, 4, 2, 16, 16, 64, 4, one, one, 12, 6, 0, None, 0, None) == -1   # pooled blocks without a window
+    assert lib.hm_attn_rows(1, one, one, one, one, one, one, None, 40, 0, 0.1, one, 4, 4, 2, 16, 16, 64, 4, one, one, 12, 5, 0, None, 0, None) == -1   # pooled pages too small
     assert lib.hm_group_norm_residual(1, one, one, None, one, None, 3, 1e-5, None, 4, 64, None) == -1     # groups do not divide the width
-    assert lib.hm_attn_decode(one, one, one, one, one, None, 0, 0, 0.1, one, 2, 4, 2, 64, 64, 64, 4, 2, one, 16, None, None, 0, 0, None) == -3  # workspace
+    assert lib.hm_attn_decode(one, one, one, one, one, None, 0, 0, 0.1, one, 2, 4, 2, 64, 64, 64, 4, 2, one, 16, None, None, 0, 0, 0, None, 0, None) == -3  # workspace
     assert b"workspace" in lib.hm_last_error()
+    assert lib.hm_attn_rows(1, one, one, one, one, one, one, None, 0, 0, 0.1, one, 4, 4, 2, 16, 16, 64, 4, None, None, 0, 0, 8, one, 0,
+                            None) == -1                                                                   # a head bias without sigmoid weights
+    assert lib.hm_attn_tiles(one, one, one, one, one, one, one, 0, 0, 0.1, one, 2, 8, 4, 2, 16, 16, 64, 4, None, None, 0, 0, 8, None, 1,
+                             None) == -1                                                                  # sigmoid weights with a sink
+    assert lib.hm_attn_rows(1, one, one, one, one, one, one, None, 9, 2, 0.1, one, 4, 4, 2, 16, 16, 64, 4, None, None, 0, 0, 8, None, 0,
+                            None) == -1                                                                   # a chunked mask with kept first tokens
+    assert lib.hm_lightning_recurrence(1, one, 40, 0, 16, 32, one, one, one, one, one, one, 2, 2, 8, 8, 1, None) == -1   # rows narrower than the columns
+    assert lib.hm_lightning_recurrence(1, one, 4096, 0, 1024, 2048, one, one, one, one, one, one, 2, 2, 512, 8, 1, None) == -2   # dim > 256
+    assert lib.hm_dyt_residual(1, one, one, None, one, None, one, None, None, None, None, 4, 64, None) == -1   # a norm without its bias
     assert lib.hm_delta_recurrence(1, one, one, 10, one, one, one, one, one, 2, 2, 8, 1, None) == -1     # v rows narrower than heads * dim
     assert lib.hm_delta_recurrence(1, one, one, 1024, one, one, one, one, one, 2, 2, 512, 1, None) == -2  # dim > 256
