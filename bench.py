@@ -402,7 +402,7 @@ def main():
                     help="instead of the headline benchmark: prefill / decode throughput of another model family (--family) "
                          "beside Qwen3 at equal layer sizes (w1024 w2048 w4096; default the first two) and the kernel-by-kernel "
                          "roofline table")
-    ap.add_argument("--family", default="pasizen", choices=["pasizen", "lipelix", "galupel"], help="the family --families measures")
+    ap.add_argument("--family", default="pasizen", choices=["pasizen", "lipelix", "galupel", "lilevik"], help="the family --families measures")
     ap.add_argument("--backend", default="nccl", choices=["nccl", "gloo"],
                     help="gloo = rehearsal of the multi-rank path on fewer GPUs than ranks (ranks share devices)")
     args = ap.parse_args()

@@ -4,7 +4,9 @@
  * token shift with a carried row per sequence, the preparation of q/k/v (projection norms, partial rotation,
  * unit-norm heads, value blending between layers, paged cache store), attention over the paged cache with
  * sinks and sliding windows that keep the first tokens, the generalized delta rule with a float32 state per
- * sequence, and squared ReLU.
+ * sequence, and squared ReLU.  Later additions: the grouped-norm and the Dynamic-Tanh residual boundaries, pooled
+ * blocks, chunked masks and sigmoid weights in the attention kernels, interleaved rotation on any frequency table and
+ * unit-RMS value heads in the preparation, and linear attention with a constant decay per head and a float32 state.
  *
  * Conventions (those of libqlinear and libseqmix): all pointers are DEVICE pointers owned by the caller,
  * matrices are row-major and dense unless a stride (in elements) is named; `stream` is a hipStream_t passed as

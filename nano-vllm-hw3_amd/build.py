@@ -5,9 +5,10 @@ Three libraries, each from its own folder of translation units, so that a model 
   seqmix   csrc/seqmix/*.hip  -> nanovllm/_lib/libseqmix.so    (multi-stream residuals, short convolutions, latent
                                                                 attention with or without a rotated part and a window,
                                                                 PolyNorm / clamped GLU / GELU experts, expert routing)
-  hymix    csrc/hymix/*.hip   -> nanovllm/_lib/libhymix.so     (gated and grouped-norm residuals, token shift, attention
-                                                                with sinks, windows and pooled blocks over a paged
-                                                                cache, delta-rule recurrence)
+  hymix    csrc/hymix/*.hip   -> nanovllm/_lib/libhymix.so     (gated, grouped-norm and tanh-norm residuals, token shift,
+                                                                attention with sinks, windows, pooled blocks, chunked
+                                                                masks and sigmoid weights over a paged cache, delta-rule
+                                                                and constant-decay recurrences)
 ``python build.py [--force] [qlinear|seqmix|hymix]`` builds one of them, or all without a name."""
 import os
 import shutil

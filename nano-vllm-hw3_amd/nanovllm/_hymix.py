@@ -1,6 +1,7 @@
 """ctypes binding of libhymix.so (the C ABI declared in include/hymix.h): scaled embedding, the gated sublayer boundary
 with norms on both sides, token shift with carried state, rotary attention over a paged key/value cache with sinks and
-windows, the generalized delta rule with its per-sequence state, squared ReLU.  No fallback on a GPU: a missing library
+windows, chunked masks and sigmoid weights, the generalized delta rule and linear attention with a constant decay with their
+per-sequence states, squared ReLU, the grouped-norm and tanh-norm residual boundaries.  No fallback on a GPU: a missing library
 raises (``build_if_missing`` compiles it in-tree first, which needs hipcc but no GPU)."""
 import ctypes
 import os

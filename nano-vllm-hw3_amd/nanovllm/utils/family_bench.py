@@ -1,7 +1,8 @@
 """Throughput of the Pasizen or the Lipelix family beside the Qwen3 decoder at equal size (random weights, bf16, one
 GPU), and the time of every libseqmix / libhymix kernel beside the like kernel of the Qwen3 path with both against their
 rooflines; for the Galupel family the comparison is with Pasizen, the closest of the three (latent attention and routed
-experts), and its kernels stand beside the forms of the same kernels that Pasizen and Lipelix run.  Used by
+experts), and its kernels stand beside the forms of the same kernels that Pasizen and Lipelix run; for the Lilevik
+family with Galupel (latent attention, masked attention, routed experts) and Lipelix (a recurrent mixer).  Used by
 ``bench.py --families [--family NAME]``; prints one JSON object."""
 import json
 import os
@@ -11,6 +12,7 @@ import time
 import torch
 
 HBM_GBPS, MFMA_TFLOPS = 8000.0, 2500.0        # MI355X: HBM3E peak, dense bf16 matrix peak
+VALU_F32_TFLOPS = 157.3                        # float32 vector peak: the bound of arithmetic that must stay float32
 
 SIZES = {                                      # name -> (width, heads, ff, layers, latent rank)
     "w1024": (1024, 16, 3072, 4, 128),
@@ -71,6 +73,23 @@ def galupel_config(width, heads, ff, layers, rank):
                 max_positions=8192, layers=specs)
 
 
+def lilevik_config(width, heads, ff, layers, rank):
+    """Lightning attention (heads of 128 x 128 over the model's width), latent attention (queries through a latent of
+    3 x rank, a 64-channel rotated part beside the key/value latent: a cache row as wide as Galupel's at the size), and two
+    grouped-head attention layers (heads / 2 key/value heads of 128, chunks of 512 positions, sigmoid weights, half of
+    every head rotated on a table stretched 4x); every layer has 16 SiLU-gated experts of ff/4 with 4 chosen."""
+    lh = max(1, width // 128)
+    light = dict(heads=lh, dim=128, vdim=128, decay=[1.0 - 2.0 ** -(3 + 6 * i / max(1, lh - 1)) for i in range(lh)])
+    lat = dict(heads=heads, dim=128, rot_dim=64, vdim=128, kv_rank=rank - 64, q_rank=3 * rank, scale=192 ** -0.5,
+               rot=dict(dims=64, base=10000.0))
+    att = dict(heads=heads, kv_heads=max(1, heads // 2), dim=128, vdim=128, scale=128 ** -0.5, mask=dict(size=512),
+               rot=dict(dims=64, base=10000.0, scaling=dict(factor=4.0, original=2048, fast=32.0, slow=1.0)))
+    moe = dict(kind="moe", expert=dict(ff=ff // 4), router=dict(experts=16, top=4))
+    kinds = [("lightning", light), ("latent_attention", lat), ("attention", att), ("attention", att)]
+    return dict(architecture="Lilevik", vocab=VOCAB, width=width, norm=dict(eps=1e-5), max_positions=8192,
+                layers=[dict(type=kinds[i % 4][0], mixer=kinds[i % 4][1], mlp=moe) for i in range(layers)])
+
+
 def _model_dir(cfg):
     d = tempfile.mkdtemp(prefix="family_bench_")
     with open(os.path.join(d, "config.json"), "w") as f:
@@ -96,7 +115,8 @@ def engine_throughput(family, size, prefill_seqs=8, prefill_len=1024, decode_seq
     width, heads, ff, layers, rank = SIZES[size]
     cfg = (pasizen_config(width, heads, ff, layers, rank) if family == "pasizen" else
            lipelix_config(width, heads, ff, layers) if family == "lipelix" else
-           galupel_config(width, heads, ff, layers, rank) if family == "galupel" else qwen3_config(width, heads, ff, layers))
+           galupel_config(width, heads, ff, layers, rank) if family == "galupel" else
+           lilevik_config(width, heads, ff, layers, rank) if family == "lilevik" else qwen3_config(width, heads, ff, layers))
     llm = LLM(_model_dir(cfg), load_format="dummy", enforce_eager=False, max_model_len=2048,
               max_num_seqs=decode_seqs, max_num_batched_tokens=prefill_seqs * prefill_len, gpu_memory_utilization=0.5)
     g = torch.Generator().manual_seed(0)
@@ -527,12 +547,179 @@ def galupel_kernel_table(width=2048, heads=16, rank=256, ff=6144, T=8192, seq=10
     return rows
 
 
+def lilevik_kernel_table(width=2048, heads=16, rank=256, ff=6144, T=8192, seq=1024, B=64, ctx=1024, chunk=512):
+    """Seconds per launch of every kernel form the Lilevik family runs at a layer's size, its bound and the fraction of it
+    reached; beside each the form of the like kernel that the closest existing family runs (`like`): Galupel's for the
+    residual boundary, attention, latent side, router and experts, Lipelix's for the recurrence."""
+    from nanovllm import hy_ops, seq_ops
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+
+    def add(name, like, sec, bytes_=0, flops=0, peak=MFMA_TFLOPS):
+        bound = max(bytes_ / (HBM_GBPS * 1e9), flops / (peak * 1e12))
+        rows.append(dict(kernel=name, like=like, us=round(sec * 1e6, 1), bound_us=round(bound * 1e6, 1),
+                         of_roofline=round(bound / sec, 3), bound="flops" if flops / (peak * 1e12) > bytes_ / (HBM_GBPS * 1e9) else "bytes"))
+    r = lambda *s: torch.randn(*s, device=dev).to(bf)  # noqa: E731
+    nseq, bs, G, D, Rd = T // seq, 64, heads // 2, 128, 64
+    R = rank - Rd
+    import numpy as np
+
+    def context(portions):
+        tables, nxt = [], 0
+        for p0, n in portions:
+            nb = (p0 + n + bs - 1) // bs
+            tables.append(list(range(nxt, nxt + nb)))
+            nxt += nb
+        tok_seq = np.concatenate([np.full(n, b) for b, (_, n) in enumerate(portions)])
+        tok_pos = np.concatenate([np.arange(p0, p0 + n) for p0, n in portions])
+        slot = np.concatenate([np.asarray(tables[b])[np.arange(p0, p0 + n) // bs] * bs + np.arange(p0, p0 + n) % bs
+                               for b, (p0, n) in enumerate(portions)])
+        mb = max(len(t) for t in tables)
+        bt = np.zeros((len(portions), mb), dtype=np.int32)
+        for b, t in enumerate(tables):
+            bt[b, :len(t)] = t
+        qs = np.concatenate([[0], np.cumsum([n for _, n in portions])])
+        i32 = lambda v: torch.tensor(np.asarray(v), dtype=torch.int32, device=dev)  # noqa: E731
+        return seq_ops.StepContext(tok_seq=i32(tok_seq), tok_pos=i32(tok_pos), qstart=i32(qs), seq_pos0=i32([p for p, _ in portions]),
+                                   ctx_lens=i32([p + n for p, n in portions]), seq_slot=i32(list(range(len(portions)))),
+                                   slot_mapping=i32(slot), block_tables=i32(bt), num_seqs=len(portions), num_tokens=int(qs[-1]),
+                                   max_q=max(n for _, n in portions), block_size=bs, qstart_host=qs.tolist()), nxt
+    pre, nblk_p = context([(0, seq)] * nseq)
+    dec, nblk_d = context([(ctx - 1, 1)] * B)
+    nblk = max(nblk_p, nblk_d)
+    # ---- residual boundary: tanh norm of the result + add + the next tanh norm | Galupel: grouped RMS norms
+    x, y = torch.randn(T, width, device=dev), r(T, width)
+    n1, n2 = (r(width), r(width), torch.rand(1, device=dev)), (r(width), r(width), torch.rand(1, device=dev))
+    add("hm_dyt_residual (T=%d)" % T, "hm_group_norm_residual", _event_time(lambda: hy_ops.dyt_residual(x, y, n1, n2, bf)),
+        bytes_=T * width * (8 + 2 + 2))
+    pw, nw = r(width), r(width)
+    add("hm_group_norm_residual (T=%d)" % T, "-", _event_time(lambda: hy_ops.group_norm_residual(x, y, pw, 4, 1e-5, bf, next_w=nw)),
+        bytes_=T * width * (8 + 2 + 2))
+    # ---- q/k/v preparation: whole-projection norms, interleaved rotation, unit-RMS values | Galupel: per-head norm + temperature
+    kc, vc = r(nblk, bs, G, D), r(nblk, bs, G, D)
+    qkv = r(T, (heads + 2 * G) * D)
+    qn, kn = r(heads * D), r(G * D)
+    inv_freq, mag = hy_ops.rotary_table(64, 1e4, dev, dict(factor=4.0, original=2048, fast=32.0, slow=1.0))
+    add("hm_qkv_prepare (T=%d, projection norm + interleaved rotation + unit values)" % T, "hm_qkv_prepare (head norm + temperature)",
+        _event_time(lambda: hy_ops.qkv_prepare(qkv, heads, G, D, D, qn, kn, 1e-5, inv_freq, False, pre, kc, vc, interleaved=True,
+                                               rot_mag=mag, v_unit_norm=True)), bytes_=T * (heads + 2 * G) * D * 4)
+    hw, temp = r(D), torch.rand(heads, device=dev) + 0.5
+    add("hm_qkv_prepare (T=%d, head norm + temperature)" % T, "-",
+        _event_time(lambda: hy_ops.qkv_prepare(qkv, heads, G, D, D, None, None, 1e-5, None, False, pre, kc, vc, None, None, hw, hw, temp)),
+        bytes_=T * (heads + 2 * G) * D * 4)
+    # ---- attention, prefill: chunked mask + sigmoid weights | Galupel: window + pooled blocks in a softmax
+    q = r(T, heads, D)
+    hb = torch.randn(heads, device=dev) - 2.0
+    cpairs = nseq * heads * sum(i % chunk + 1 for i in range(seq))
+    add("hm_attn_tiles chunk %d, sigmoid (%dx%d)" % (chunk, nseq, seq), "hm_attn_tiles window + pooled",
+        _event_time(lambda: hy_ops.paged_attention(q, kc, vc, pre, 0.09, chunk=chunk, sigmoid=True, head_bias=hb), 5), flops=cpairs * 4 * D)
+    pool = 64
+    pr = hy_ops.pool_rows_per_page(bs, pool)
+    kp, vp = r(nblk, pr, G, D), r(nblk, pr, G, D)
+    wpairs = nseq * heads * sum(min(i + 1, chunk) + max(0, (i + 1 - chunk) // pool) for i in range(seq))
+    add("hm_attn_tiles window %d + pooled %d (%dx%d)" % (chunk, pool, nseq, seq), "-",
+        _event_time(lambda: hy_ops.paged_attention(q, kc, vc, pre, 0.09, None, chunk, 0, pooled=(kp, vp, pool)), 5), flops=wpairs * 4 * D)
+    # ---- attention, decode
+    qd = r(B, heads, D)
+    in_chunk = (ctx - 1) % chunk + 1
+    add("hm_attn_decode chunk %d, sigmoid (B=%d, ctx=%d: %d keys)" % (chunk, B, ctx, in_chunk), "hm_attn_decode window + pooled",
+        _event_time(lambda: hy_ops.paged_attention(qd, kc, vc, dec, 0.09, chunk=chunk, sigmoid=True, head_bias=hb)),
+        bytes_=B * in_chunk * G * D * 4)
+    seen = max(0, (ctx - chunk) // pool)
+    add("hm_attn_decode window %d + pooled %d (B=%d, ctx=%d)" % (chunk, pool, B, ctx), "-",
+        _event_time(lambda: hy_ops.paged_attention(qd, kc, vc, dec, 0.09, None, chunk, 0, pooled=(kp, vp, pool))),
+        bytes_=B * (chunk + seen) * G * D * 4)
+    # ---- lightning recurrence | Lipelix: delta rule (heads of 64 over the width).  Both states are float32 by design, so the
+    # arithmetic of a step (4 D V flops per token and head here, 10 D^2 there) is priced at the float32 vector peak
+    LH = width // 128
+    proj = r(T, 4 * LH * 128)
+    decay = torch.rand(LH, device=dev) * 0.1 + 0.9
+    state = torch.zeros(max(nseq, B), LH, 128, 128, device=dev)
+    add("hm_lightning_recurrence prefill (%dx%d, %d heads of 128x128)" % (nseq, seq, LH), "hm_delta_recurrence prefill",
+        _event_time(lambda: hy_ops.lightning_recurrence(proj, 0, LH * 128, 2 * LH * 128, LH, 128, 128, decay, state, pre), 5),
+        bytes_=T * LH * 128 * (3 * 2 + 4) + nseq * LH * 128 * 128 * 8, flops=T * LH * 4 * 128 * 128, peak=VALU_F32_TFLOPS)
+    projd = proj[:B].contiguous()
+    add("hm_lightning_recurrence decode (B=%d)" % B, "hm_delta_recurrence decode",
+        _event_time(lambda: hy_ops.lightning_recurrence(projd, 0, LH * 128, 2 * LH * 128, LH, 128, 128, decay, state, dec)),
+        bytes_=B * LH * 128 * 128 * 8)
+    DH = width // 64
+    prep, vd = torch.rand(T, DH, 5, 64, device=dev), r(T, DH * 64)
+    dstate = torch.zeros(max(nseq, B), DH, 64, 64, device=dev)
+    add("hm_delta_recurrence prefill (%dx%d, %d heads of 64)" % (nseq, seq, DH), "-",
+        _event_time(lambda: hy_ops.delta_recurrence(prep, vd, dstate, pre), 3), bytes_=T * DH * 64 * (5 * 4 + 2 + 4) + nseq * DH * 64 * 64 * 8,
+        flops=T * DH * 10 * 64 * 64, peak=VALU_F32_TFLOPS)
+    prepd, vdd = prep[:B].contiguous(), vd[:B].contiguous()
+    add("hm_delta_recurrence decode (B=%d)" % B, "-", _event_time(lambda: hy_ops.delta_recurrence(prepd, vdd, dstate, dec)),
+        bytes_=B * DH * 64 * 64 * 8)
+    o, gcol, ow = torch.randn(T, LH, 128, device=dev), r(T, LH * 128), r(LH * 128)
+    add("hm_delta_gate_norm over all heads (T=%d)" % T, "hm_delta_gate_norm per head",
+        _event_time(lambda: hy_ops.delta_gate_norm(o.view(T, 1, LH * 128), gcol, ow, 1e-5, bf)), bytes_=T * LH * 128 * (4 + 2 + 2))
+    add("hm_delta_gate_norm per head (T=%d)" % T, "-", _event_time(lambda: hy_ops.delta_gate_norm(o, gcol, ow, 1e-5, bf)),
+        bytes_=T * LH * 128 * (4 + 2 + 2))
+    # ---- latent side: the query latent's norm; norm + rotation + store; attention without a window | Galupel: window 512
+    Q = 3 * rank
+    cache = r(nblk, bs, rank)
+    first = r(T, Q + rank)
+    qw = r(Q)
+    add("sm_rms_norm_rows query latent (T=%d, %d)" % (T, Q), "sm_latent_norm_store",
+        _event_time(lambda: seq_ops.rms_norm_rows(first[:, :Q], qw, 1e-5)), bytes_=T * Q * 4)
+    lw, cache_r = r(R), r(nblk, bs, R)
+    add("sm_latent_norm_store (T=%d)" % T, "-",
+        _event_time(lambda: seq_ops.latent_norm_store(first[:, Q:Q + R], lw, 1e-5, cache_r, pre.slot_mapping)), bytes_=T * R * 4)
+    q2, qa = r(T, heads * (D + Rd)), r(T, heads, rank)
+    rf = hy_ops.rotary_inv_freq(64, 1e4, dev)
+    add("sm_latent_rope_store (T=%d, H=%d)" % (T, heads), "(the same form as Galupel's)",
+        _event_time(lambda: seq_ops.latent_rope_store(first[:, Q:], lw, 1e-5, q2, qa, rf, Rd, heads, D, R, Rd, cache, pre)),
+        bytes_=T * (rank * 4 + heads * Rd * 4))
+    pairs = nseq * seq * (seq + 1) / 2 * heads
+    add("sm_latent_attn_tiles full, row %d+%d (%dx%d, H=%d)" % (R, Rd, nseq, seq, heads), "sm_latent_attn_tiles window",
+        _event_time(lambda: seq_ops.latent_attention(qa, cache, pre, 0.09, value_cols=R), 5), flops=pairs * 2 * (rank + R))
+    lpairs = nseq * heads * sum(min(i + 1, chunk) for i in range(seq))
+    add("sm_latent_attn_tiles window %d, row %d+%d" % (chunk, R, Rd), "-",
+        _event_time(lambda: seq_ops.latent_attention(qa, cache, pre, 0.09, value_cols=R, window=chunk), 5), flops=lpairs * 2 * (rank + R))
+    qad = r(B, heads, rank)
+    add("sm_latent_attn_decode full, row %d+%d (B=%d, ctx=%d)" % (R, Rd, B, ctx), "sm_latent_attn_decode window",
+        _event_time(lambda: seq_ops.latent_attention(qad, cache, dec, 0.09, value_cols=R)), bytes_=B * ctx * rank * 2)
+    add("sm_latent_attn_decode window %d, row %d+%d" % (chunk, R, Rd), "-",
+        _event_time(lambda: seq_ops.latent_attention(qad, cache, dec, 0.09, value_cols=R, window=chunk)), bytes_=B * chunk * rank * 2)
+    # ---- router and experts: biased logits, softmax over the chosen, SiLU-gated experts | Galupel: sigmoid + correction, GELU
+    E, top, F = 16, 4, ff // 4
+    h = r(T, width)
+    rw, rb = torch.randn(E, width, device=dev), torch.randn(E, device=dev) * 0.1
+    add("sm_moe_route softmax + bias (T=%d, E=%d)" % (T, E), "sm_moe_route sigmoid + correction",
+        _event_time(lambda: seq_ops.moe_route(h, rw, top, bias=rb)), bytes_=T * width * 2)
+    add("sm_moe_route sigmoid + correction (T=%d, E=%d)" % (T, E), "-",
+        _event_time(lambda: seq_ops.moe_route(h, rw, top, 4, 2, seq_ops.ROUTE_SIGMOID, rb, 2, False)), bytes_=T * width * 2)
+    idx, wts = seq_ops.moe_route(h, rw, top, bias=rb)
+    w_up, w_gu, w_down = r(E, F, width), r(E, 2 * F, width), r(E, width, F)
+    t_gelu = (seq_ops.tile_expert_weights(w_up, 1), seq_ops.tile_expert_weights(w_down))
+    t_glu = (seq_ops.tile_expert_weights(w_gu, 2), t_gelu[1])
+    inf = float("inf")
+    add("sm_moe_tiles128 SiLU-gated experts (T=%d, top %d of %d, F=%d)" % (T, top, E, F), "sm_moe_tiles128 GELU experts",
+        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_gu, w_down, inf, 1.0, form="tiles128", tiled=t_glu, act_kind=seq_ops.ACT_SILU_GLU), 5),
+        flops=T * top * 6 * width * F)
+    add("sm_moe_tiles128 GELU experts (T=%d)" % T, "-",
+        _event_time(lambda: seq_ops.moe_experts(h, idx, wts, w_up, w_down, 0.0, form="tiles128", tiled=t_gelu, act_kind=seq_ops.ACT_GELU), 5),
+        flops=T * top * 4 * width * F)
+    hd = h[:B].contiguous()
+    idx_d, wts_d = seq_ops.moe_route(hd, rw, top, bias=rb)
+    touched = len(torch.unique(idx_d))
+    add("sm_moe_grouped SiLU-gated experts (T=%d: decode)" % B, "sm_moe_grouped GELU experts",
+        _event_time(lambda: seq_ops.moe_experts(hd, idx_d, wts_d, w_gu, w_down, inf, 1.0, form="grouped", tiled=t_glu, act_kind=seq_ops.ACT_SILU_GLU)),
+        bytes_=touched * 3 * F * width * 2)
+    add("sm_moe_grouped GELU experts (T=%d: decode)" % B, "-",
+        _event_time(lambda: seq_ops.moe_experts(hd, idx_d, wts_d, w_up, w_down, 0.0, form="grouped", tiled=t_gelu, act_kind=seq_ops.ACT_GELU)),
+        bytes_=touched * 2 * F * width * 2)
+    return rows
+
+
 def main(sizes=("w1024", "w2048"), kernels=True, family="pasizen"):
     out = dict(metric="family comparison", dtype="bf16", data="synthetic (random weights)", throughput=[], kernels=[])
+    beside = {"galupel": ("pasizen", "qwen3"), "lilevik": ("galupel", "lipelix", "qwen3")}.get(family, ("qwen3",))
     for size in sizes:
-        for fam in ((family, "pasizen", "qwen3") if family == "galupel" else (family, "qwen3")):
+        for fam in (family,) + beside:
             out["throughput"].append(engine_throughput(fam, size))
     if kernels:
-        out["kernels"] = (kernel_table() if family == "pasizen" else galupel_kernel_table() if family == "galupel" else
-                          hymix_kernel_table())
+        out["kernels"] = {"pasizen": kernel_table, "galupel": galupel_kernel_table, "lilevik": lilevik_kernel_table}.get(
+            family, hymix_kernel_table)()
     return out
