@@ -15,7 +15,8 @@ __device__ __forceinline__ float lt_sum8(float v) {       // sum over 8 neighbou
     return v;
 }
 
-__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+// z sigmoid(z) from the hardware's exponential and reciprocal (float32, a few units in the last place)
+__device__ __forceinline__ float silu_f(float z) { return z * __builtin_amdgcn_rcpf(1.f + __expf(-z)); }
 
 // One workgroup of 256 threads per (sequence, head, 32 CV value channels).  A thread keeps CV neighbouring columns of S
 // (value channels) over DK / 8 key channels in registers: a column (DK >= D key channels) is spread over 8 neighbouring
@@ -49,25 +50,35 @@ __global__ __launch_bounds__(256) void lightning_kernel(const T* __restrict__ pr
 #pragma unroll
         for (int c = 0; c < CV; ++c) s[ii][c] = (!fresh && j0 + c < V && i < D) ? st[(size_t)i * V + j0 + c] : 0.f;
     }
-    // the loaded values stay untouched in registers until they are deposited (silu(0) = 0 keeps the padding zero): nothing
-    // waits for global memory before the current chunk's tokens have run
+    // Which value of a chunk a thread fetches does not change from chunk to chunk: its column in the row and its token
+    // inside the chunk are worked out once (column -1: padding).  The loaded values stay untouched in registers until they
+    // are deposited (silu(0) = 0 keeps the padding zero): nothing waits for global memory before the current chunk's tokens
+    // have run.
+    int col_of[NR], tok_of[NR];
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+        const int e = tid + 256 * k;
+        const int tc = e / TOK, rem = e - tc * TOK;
+        int c = -1;
+        if (e < CH * TOK) {
+            if (rem < 2 * DK) {
+                const int part = rem / DK, i = rem - part * DK;
+                if (i < D) c = (part ? k_off : q_off) + hd * D + i;
+            } else {
+                const int jj = blockIdx.z * COLS + (rem - 2 * DK);
+                if (jj < V) c = v_off + hd * V + jj;
+            }
+        }
+        col_of[k] = c;
+        tok_of[k] = tc;
+    }
     T regs[NR];
     auto request = [&](int tok0) {
 #pragma unroll
         for (int k = 0; k < NR; ++k) {
-            const int e = tid + 256 * k;
-            const int tc = e / TOK, rem = e - tc * TOK, tok = tok0 + tc;
+            const int tok = tok0 + tok_of[k];
             T val = from_f<T>(0.f);
-            if (e < CH * TOK && tok < n) {
-                const T* row = proj + (size_t)(q0 + tok) * row_stride;
-                if (rem < 2 * DK) {
-                    const int part = rem / DK, i = rem - part * DK;
-                    if (i < D) val = row[(part ? k_off : q_off) + hd * D + i];
-                } else {
-                    const int jj = blockIdx.z * COLS + (rem - 2 * DK);
-                    if (jj < V) val = row[v_off + hd * V + jj];
-                }
-            }
+            if (col_of[k] >= 0 && tok < n) val = proj[(size_t)(q0 + tok) * row_stride + col_of[k]];
             regs[k] = val;
         }
     };
