@@ -46,12 +46,12 @@ class LilevikLayer(nn.Module):
                                          rot_dim=m.get("rot_dim", 0), rot_dims=rot.get("dims", 0), rot_base=rot.get("base", 10000.0),
                                          q_rank=m.get("q_rank", 0))
         elif self.kind == "attention":
-            self.mixer = PagedRotaryAttention(W, m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"], eps,
-                                              rot.get("dims", 0), rot.get("base", 10000.0), proj_norm=True, interleaved=True,
+            self.mixer = PagedRotaryAttention(W, m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"]),
+                                              m["scale"], eps, rot.get("dims", 0), rot.get("base", 10000.0), proj_norm=True, interleaved=True,
                                               rot_scaling=rot.get("scaling"), v_unit_norm=True,
                                               chunk=(m.get("mask") or {}).get("size", 0), weights="sigmoid")
         elif self.kind == "lightning":
-            self.mixer = LightningAttention(W, m["heads"], m["dim"], m["vdim"], m["decay"], eps)
+            self.mixer = LightningAttention(W, m["heads"], m["dim"], m.get("vdim", m["dim"]), m["decay"], eps)
         else:
             raise ValueError(f"unknown mixer type {self.kind!r}")
         mlp = spec.get("mlp")
@@ -166,9 +166,9 @@ class LilevikForCausalLM(nn.Module):
             p, m = f"l{i}.", spec["mixer"]
             norm(t, p + "norm1")
             norm(t, p + "norm1b")
-            H, D, V = m["heads"], m["dim"], m["vdim"]
+            H, D, V = m["heads"], m["dim"], m.get("vdim", m["dim"])
             if spec["type"] == "attention":
-                G = m["kv_heads"]
+                G = m.get("kv_heads", H)
                 t.update({p + "mix.q": rnd(H * D, W, s=W ** -0.5), p + "mix.k": rnd(G * D, W, s=W ** -0.5),
                           p + "mix.v": rnd(G * V, W, s=W ** -0.5), p + "mix.q.norm": 1 + rnd(H * D, s=0.2),
                           p + "mix.k.norm": 1 + rnd(G * D, s=0.2), p + "mix.pb": rnd(H, s=1.0) - 2.0,
